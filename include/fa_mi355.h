@@ -1,0 +1,108 @@
+/*
+ * fa_mi355.h -- C ABI of libfa_mi355.so: flash attention forward/backward with an optional
+ * materialized bias for AMD MI355X (gfx950).
+ *
+ * The two launch entry points replace the host launchers of the reference one for one:
+ *   fa_fwd  <->  _flash_attn_fwd(q, k, v, bias, causal, sm_scale) -> (o, M)
+ *                /root/reference/flash_attention.py:649-685
+ *   fa_bwd  <->  _flash_attn_bwd(do, q, k, v, o, bias, causal, sm_scale, M, dq, dk, dv, dbias)
+ *                /root/reference/flash_attention.py:688-763
+ * Like them, the library owns no memory: every buffer (including the backward workspace) is
+ * allocated by the caller, every call only enqueues work on the stream it is given and returns
+ * without synchronizing.  All entry points are re-entrant and keep no mutable global state.
+ *
+ * Layouts (element strides, as the reference passes them, flash_attention.py:670-675):
+ *   q, o, do, dq : (B, M, H, D)     k, v, dk, dv : (B, N, H, D)     the D stride must be 1
+ *   bias, dbias  : (B, H, M, N)     any strides, 0 included (an expanded mask works as is)
+ *   lse, delta   : (B, H, M) fp32, dense, in log2 units: lse = log2(sum_j 2^(s_ij))
+ * Base pointers of q/k/v/o/do/dq/dk/dv and their B/seq/H strides must be multiples of 16 bytes
+ * (FA_ERR_LAYOUT otherwise); bias/dbias have no alignment requirement, but rows with unit N
+ * stride and 16-byte aligned row starts take the fast path.
+ */
+#ifndef FA_MI355_H
+#define FA_MI355_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FA_ABI_VERSION 1
+
+/* element type of q, k, v, o and their gradients */
+enum fa_dtype { FA_F16 = 0, FA_BF16 = 1 };
+
+/* element type of bias (and of dbias, which always has the type of bias);
+ * FA_BIAS_BOOL is one byte per element, non-zero = keep (flash_attention.py:48-50) */
+enum fa_bias_dtype { FA_BIAS_NONE = 0, FA_BIAS_BOOL = 1, FA_BIAS_F16 = 2, FA_BIAS_BF16 = 3, FA_BIAS_F32 = 4 };
+
+enum fa_status {
+    FA_OK = 0,
+    FA_ERR_NULL = -1,        /* a required pointer is NULL */
+    FA_ERR_SHAPE = -2,       /* a dimension is < 1, or causal with M != N */
+    FA_ERR_HEAD_DIM = -3,    /* D not in {16, 32, 64, 128, 256}  (flash_attention.py:776) */
+    FA_ERR_DTYPE = -4,       /* unknown dtype / bias dtype, or dbias requested for a bool bias */
+    FA_ERR_LAYOUT = -5,      /* alignment or stride rule above violated */
+    FA_ERR_WORKSPACE = -6,   /* workspace NULL or smaller than fa_bwd_workspace_bytes() */
+    FA_ERR_UNSUPPORTED = -7, /* combination not built into this library */
+    FA_ERR_LAUNCH = -8       /* the HIP runtime rejected a launch (hipGetLastError) */
+};
+
+/* Problem description shared by forward and backward.  Strides are in elements. */
+typedef struct fa_problem {
+    int32_t B, H, M, N, D;
+    int32_t dtype;       /* enum fa_dtype */
+    int32_t bias_dtype;  /* enum fa_bias_dtype */
+    int32_t causal;      /* 0 / 1; top-left aligned, requires M == N (flash_attention.py:45,777) */
+    float sm_scale;      /* scores = (q . k) * sm_scale + bias  (flash_attention.py:149-150) */
+} fa_problem;
+
+/* _flash_attn_fwd: flash_attention.py:649-685.  o and lse are outputs. */
+typedef struct fa_fwd_args {
+    fa_problem p;
+    const void *q, *k, *v, *bias; /* bias may be NULL iff bias_dtype == FA_BIAS_NONE */
+    void *o;
+    float *lse;                   /* (B, H, M) */
+    int64_t q_strides[4], k_strides[4], v_strides[4], o_strides[4]; /* (B, seq, H, D) */
+    int64_t bias_strides[4];      /* (B, H, M, N) */
+} fa_fwd_args;
+
+/* _flash_attn_bwd: flash_attention.py:688-763.  dq, dk, dv (and dbias when non-NULL, i.e. when
+ * the bias is trainable, flash_attention.py:693,799) are outputs and are fully overwritten:
+ * unlike the reference's dbias they need no zero fill by the caller. */
+typedef struct fa_bwd_args {
+    fa_problem p;
+    const void *q, *k, *v, *o, *dout, *bias;
+    const float *lse;             /* as written by fa_fwd */
+    void *dq, *dk, *dv, *dbias;   /* dbias NULL = bias not trainable */
+    void *workspace;              /* fa_bwd_workspace_bytes() bytes, 256-byte aligned */
+    size_t workspace_bytes;
+    int64_t q_strides[4], k_strides[4], v_strides[4], o_strides[4], do_strides[4];
+    int64_t dq_strides[4], dk_strides[4], dv_strides[4];
+    int64_t bias_strides[4], dbias_strides[4];
+} fa_bwd_args;
+
+/* Version of this header the library was built against (== FA_ABI_VERSION). */
+int fa_abi_version(void);
+
+/* Static, NUL-terminated description of a status code. */
+const char *fa_strerror(int status);
+
+/* Enqueue the forward on `stream` (a hipStream_t passed as void*; NULL = the null stream).
+ * Replaces _flash_attn_fwd, flash_attention.py:649-685 (bias pre-scale :660-663 included). */
+int fa_fwd(const fa_fwd_args *args, void *stream);
+
+/* Bytes of scratch the backward needs for this problem: delta (flash_attention.py:689) plus the
+ * fp32 dQ accumulator.  Depends on B, H, M, D only. */
+size_t fa_bwd_workspace_bytes(const fa_problem *p);
+
+/* Enqueue the backward (delta, dK/dV/dBias/dQ) on `stream`.
+ * Replaces _flash_attn_bwd, flash_attention.py:688-763 (K and bias pre-scale :699-704 included). */
+int fa_bwd(const fa_bwd_args *args, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FA_MI355_H */

@@ -1,0 +1,158 @@
+// C ABI of libfa_mi355.so (declared in include/fa_mi355.h): argument validation and dispatch.
+// Host code only; the kernels live in fa_fwd.hip and fa_bwd.hip.
+#include <hip/hip_runtime.h>
+
+#include "../../include/fa_mi355.h"
+#include "fa_params.hpp"
+
+namespace fa {
+hipError_t launch_fwd(const FwdParams& p, int D, int dtype, int bias, bool causal, hipStream_t st);
+hipError_t launch_bwd(const BwdParams& p, int D, int dtype, int bias, bool causal, bool dbias, hipStream_t st);
+int fwd_block_m();
+int bwd_block_n(int D);
+}  // namespace fa
+
+namespace {
+
+bool head_dim_ok(int d) { return d == 16 || d == 32 || d == 64 || d == 128 || d == 256; }
+
+int check_problem(const fa_problem& p) {
+    if (p.B < 1 || p.H < 1 || p.M < 1 || p.N < 1) return FA_ERR_SHAPE;
+    if (!head_dim_ok(p.D)) return FA_ERR_HEAD_DIM;
+    if (p.dtype != FA_F16 && p.dtype != FA_BF16) return FA_ERR_DTYPE;
+    if (p.bias_dtype < FA_BIAS_NONE || p.bias_dtype > FA_BIAS_F32) return FA_ERR_DTYPE;
+    if (p.causal && p.M != p.N) return FA_ERR_SHAPE;
+    // a grid is one-dimensional: tiles * B * H must fit in 31 bits
+    if ((int64_t)((p.M + 63) / 64 + (p.N + 63) / 64) * p.B * p.H >= (1ll << 31)) return FA_ERR_SHAPE;
+    return FA_OK;
+}
+
+// 16-byte rule for a (B, seq, H, D) tensor of 2-byte elements; strides of extent-1 dims are free
+bool qkv_layout_ok(const void* ptr, const int64_t s[4], int nb, int ns, int nh) {
+    if (s[3] != 1) return false;
+    if (reinterpret_cast<uintptr_t>(ptr) % 16 != 0) return false;
+    if (nb > 1 && s[0] % 8 != 0) return false;
+    if (ns > 1 && s[1] % 8 != 0) return false;
+    if (nh > 1 && s[2] % 8 != 0) return false;
+    return true;
+}
+
+fa::Strides3 s3(const int64_t s[4]) { return fa::Strides3{s[0], s[1], s[2]}; }
+fa::Strides4 s4(const int64_t s[4]) { return fa::Strides4{s[0], s[1], s[2], s[3]}; }
+
+int bias_elem_size(int bias_dtype) {
+    switch (bias_dtype) {
+        case FA_BIAS_BOOL: return 1;
+        case FA_BIAS_F16:
+        case FA_BIAS_BF16: return 2;
+        case FA_BIAS_F32: return 4;
+    }
+    return 0;
+}
+
+// rows of bias may be fetched with aligned 16-byte loads
+bool bias_vec_ok(const void* ptr, const int64_t s[4], const fa_problem& p) {
+    int es = bias_elem_size(p.bias_dtype);
+    if (es == 0) return false;
+    if (p.N > 1 && s[3] != 1) return false;
+    if (reinterpret_cast<uintptr_t>(ptr) % 16 != 0) return false;
+    if (p.B > 1 && (s[0] * es) % 16 != 0) return false;
+    if (p.H > 1 && (s[1] * es) % 16 != 0) return false;
+    if (p.M > 1 && (s[2] * es) % 16 != 0) return false;
+    return true;
+}
+
+size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+}  // namespace
+
+extern "C" {
+
+int fa_abi_version(void) { return FA_ABI_VERSION; }
+
+const char* fa_strerror(int status) {
+    switch (status) {
+        case FA_OK: return "ok";
+        case FA_ERR_NULL: return "a required pointer is NULL";
+        case FA_ERR_SHAPE: return "bad shape: a dimension is < 1, too large, or causal with M != N";
+        case FA_ERR_HEAD_DIM: return "head dimension must be one of 16, 32, 64, 128, 256";
+        case FA_ERR_DTYPE: return "unsupported dtype / bias dtype (or dbias requested for a bool bias)";
+        case FA_ERR_LAYOUT: return "layout: head-dim stride must be 1 and pointers/strides 16-byte aligned";
+        case FA_ERR_WORKSPACE: return "workspace is NULL, misaligned or smaller than fa_bwd_workspace_bytes()";
+        case FA_ERR_UNSUPPORTED: return "combination not built into this library";
+        case FA_ERR_LAUNCH: return "HIP kernel launch failed";
+    }
+    return "unknown status";
+}
+
+int fa_fwd(const fa_fwd_args* a, void* stream) {
+    if (!a) return FA_ERR_NULL;
+    const fa_problem& p = a->p;
+    int st = check_problem(p);
+    if (st != FA_OK) return st;
+    if (!a->q || !a->k || !a->v || !a->o || !a->lse) return FA_ERR_NULL;
+    if ((p.bias_dtype != FA_BIAS_NONE) != (a->bias != nullptr)) return FA_ERR_NULL;
+    if (!qkv_layout_ok(a->q, a->q_strides, p.B, p.M, p.H) || !qkv_layout_ok(a->k, a->k_strides, p.B, p.N, p.H) ||
+        !qkv_layout_ok(a->v, a->v_strides, p.B, p.N, p.H) || !qkv_layout_ok(a->o, a->o_strides, p.B, p.M, p.H))
+        return FA_ERR_LAYOUT;
+
+    fa::FwdParams k{};
+    k.q = a->q; k.k = a->k; k.v = a->v; k.bias = a->bias; k.o = a->o; k.lse = a->lse;
+    k.sq = s3(a->q_strides); k.sk = s3(a->k_strides); k.sv = s3(a->v_strides); k.so = s3(a->o_strides);
+    k.B = p.B; k.H = p.H; k.M = p.M; k.N = p.N;
+    k.sm_scale = p.sm_scale;
+    if (a->bias) {
+        k.sbias = s4(a->bias_strides);
+        k.bias_vec = bias_vec_ok(a->bias, a->bias_strides, p) ? 1 : 0;
+    }
+    k.n_mtiles = (p.M + fa::fwd_block_m() - 1) / fa::fwd_block_m();
+    hipError_t e = fa::launch_fwd(k, p.D, p.dtype, p.bias_dtype, p.causal != 0, static_cast<hipStream_t>(stream));
+    if (e == hipErrorNotSupported) return FA_ERR_UNSUPPORTED;
+    return e == hipSuccess ? FA_OK : FA_ERR_LAUNCH;
+}
+
+size_t fa_bwd_workspace_bytes(const fa_problem* p) {
+    if (!p || check_problem(*p) != FA_OK) return 0;
+    size_t rows = (size_t)p->B * p->H * p->M;
+    return align256(rows * sizeof(float)) + align256(rows * p->D * sizeof(float));
+}
+
+int fa_bwd(const fa_bwd_args* a, void* stream) {
+    if (!a) return FA_ERR_NULL;
+    const fa_problem& p = a->p;
+    int st = check_problem(p);
+    if (st != FA_OK) return st;
+    if (!a->q || !a->k || !a->v || !a->o || !a->dout || !a->lse || !a->dq || !a->dk || !a->dv) return FA_ERR_NULL;
+    if ((p.bias_dtype != FA_BIAS_NONE) != (a->bias != nullptr)) return FA_ERR_NULL;
+    if (a->dbias && (p.bias_dtype == FA_BIAS_NONE || p.bias_dtype == FA_BIAS_BOOL)) return FA_ERR_DTYPE;
+    if (!qkv_layout_ok(a->q, a->q_strides, p.B, p.M, p.H) || !qkv_layout_ok(a->k, a->k_strides, p.B, p.N, p.H) ||
+        !qkv_layout_ok(a->v, a->v_strides, p.B, p.N, p.H) || !qkv_layout_ok(a->o, a->o_strides, p.B, p.M, p.H) ||
+        !qkv_layout_ok(a->dout, a->do_strides, p.B, p.M, p.H) || !qkv_layout_ok(a->dq, a->dq_strides, p.B, p.M, p.H) ||
+        !qkv_layout_ok(a->dk, a->dk_strides, p.B, p.N, p.H) || !qkv_layout_ok(a->dv, a->dv_strides, p.B, p.N, p.H))
+        return FA_ERR_LAYOUT;
+    size_t need = fa_bwd_workspace_bytes(&p);
+    if (!a->workspace || a->workspace_bytes < need || reinterpret_cast<uintptr_t>(a->workspace) % 256 != 0)
+        return FA_ERR_WORKSPACE;
+
+    fa::BwdParams k{};
+    k.q = a->q; k.k = a->k; k.v = a->v; k.o = a->o; k.dout = a->dout; k.bias = a->bias; k.lse = a->lse;
+    k.dq = a->dq; k.dk = a->dk; k.dv = a->dv; k.dbias = a->dbias;
+    size_t rows = (size_t)p.B * p.H * p.M;
+    k.delta = static_cast<float*>(a->workspace);
+    k.dq_acc = reinterpret_cast<float*>(static_cast<char*>(a->workspace) + align256(rows * sizeof(float)));
+    k.sq = s3(a->q_strides); k.sk = s3(a->k_strides); k.sv = s3(a->v_strides); k.so = s3(a->o_strides);
+    k.sdo = s3(a->do_strides); k.sdq = s3(a->dq_strides); k.sdk = s3(a->dk_strides); k.sdv = s3(a->dv_strides);
+    if (a->bias) k.sbias = s4(a->bias_strides);
+    if (a->dbias) k.sdbias = s4(a->dbias_strides);
+    k.B = p.B; k.H = p.H; k.M = p.M; k.N = p.N;
+    k.sm_scale = p.sm_scale;
+    int bn = fa::bwd_block_n(p.D);
+    if (bn <= 0) return FA_ERR_UNSUPPORTED;
+    k.n_ntiles = (p.N + bn - 1) / bn;
+    hipError_t e = fa::launch_bwd(k, p.D, p.dtype, p.bias_dtype, p.causal != 0, a->dbias != nullptr,
+                                  static_cast<hipStream_t>(stream));
+    if (e == hipErrorNotSupported) return FA_ERR_UNSUPPORTED;
+    return e == hipSuccess ? FA_OK : FA_ERR_LAUNCH;
+}
+
+}  // extern "C"

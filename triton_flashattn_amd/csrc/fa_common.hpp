@@ -1,0 +1,123 @@
+// Device-side building blocks shared by the gfx950 attention kernels.
+//
+// Wave = 64 lanes.  All matrix products use v_mfma_f32_32x32x16_{bf16,f16}:
+//   A (32 x 16): lane l holds row l%32, k = 8*(l/32) .. 8*(l/32)+7
+//   B (16 x 32): lane l holds col l%32, k = 8*(l/32) .. 8*(l/32)+7
+//   C (32 x 32): lane l holds col l%32; register i holds row 8*(i/4) + 4*(l/32) + i%4
+// Only the pairing of A's and B's k slots matters to the product, so operands taken from a C
+// fragment (registers 8j..8j+7 = rows {16j + 4g + 0..3, 16j + 8 + 4g + 0..3}, g = l/32) are
+// matched by loading the other operand with the same k order.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace fa {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x2 __attribute__((ext_vector_type(2)));
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kMask = -1.0e6f;  // additive mask term, in log2 units
+
+template <typename T> struct VecOf;
+template <> struct VecOf<__bf16> { typedef bf16x8 v8; typedef bf16x4 v4; };
+template <> struct VecOf<_Float16> { typedef f16x8 v8; typedef f16x4 v4; };
+
+__device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ f32x16 mfma32(f16x8 a, f16x8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+}
+
+template <typename V> __device__ __forceinline__ V as_vec(i32x4 x) { return __builtin_bit_cast(V, x); }
+template <typename V> __device__ __forceinline__ i32x4 as_raw(V x) { return __builtin_bit_cast(i32x4, x); }
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+// Value of `x` held by lane l ^ 32.
+__device__ __forceinline__ float partner32(float x) {
+    int xi = __builtin_bit_cast(int, x);
+    auto r = __builtin_amdgcn_permlane32_swap(xi, xi, false, false);
+    int other = (threadIdx.x & 32) ? r[0] : r[1];
+    return __builtin_bit_cast(float, other);
+}
+// max / sum over the lane pair {l, l ^ 32}
+__device__ __forceinline__ float pair_max(float x) {
+    int xi = __builtin_bit_cast(int, x);
+    auto r = __builtin_amdgcn_permlane32_swap(xi, xi, false, false);
+    return fmaxf(__builtin_bit_cast(float, (int)r[0]), __builtin_bit_cast(float, (int)r[1]));
+}
+__device__ __forceinline__ float pair_sum(float x) {
+    int xi = __builtin_bit_cast(int, x);
+    auto r = __builtin_amdgcn_permlane32_swap(xi, xi, false, false);
+    return __builtin_bit_cast(float, (int)r[0]) + __builtin_bit_cast(float, (int)r[1]);
+}
+
+// ---- LDS access ---------------------------------------------------------------------------
+__device__ __forceinline__ i32x4 lds_read16(const void* p) { return *reinterpret_cast<const i32x4*>(p); }
+__device__ __forceinline__ void lds_write16(void* p, i32x4 v) { *reinterpret_cast<i32x4*>(p) = v; }
+
+// ds_read_b64_tr_b16.  Within each group of 16 lanes, lane s supplies the address of four
+// consecutive 16-bit elements: row s/4, columns 4*(s%4) .. 4*(s%4)+3 of a 4 x 16 matrix.  Lane i
+// of the group receives column i of that matrix (4 values, rows 0..3).
+__device__ __forceinline__ i16x4 lds_read_tr4(const void* p) {
+    typedef i16x4 __attribute__((address_space(3))) * lds_ptr;
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p));
+}
+// Address a lane must supply so that a 32-lane half of the wave reads a 4-row x 32-column
+// block (16-bit elements, `stride` elements between rows) and lane l ends up with column l%32:
+// returns the element offset of (row0 + (l%16)/4, col0 + 16*((l/16)%2) + 4*(l%4)).
+__device__ __forceinline__ int tr_offset(int lane, int row0, int col0, int stride) {
+    int s = lane & 15;
+    return (row0 + (s >> 2)) * stride + col0 + ((lane >> 4) & 1) * 16 + (s & 3) * 4;
+}
+// 8 k-slots of an A/B operand gathered down a column of a row-major LDS tile: rows
+// row0 + 4g + {0..3} and row0 + 8 + 4g + {0..3} (g = lane/32), column col0 + lane%32.
+template <typename V8, typename T>
+__device__ __forceinline__ V8 lds_read_col8(const T* tile, int lane, int row0, int col0, int stride) {
+    int g = lane >> 5;
+    i16x4 lo = lds_read_tr4(tile + tr_offset(lane, row0 + 4 * g, col0, stride));
+    i16x4 hi = lds_read_tr4(tile + tr_offset(lane, row0 + 8 + 4 * g, col0, stride));
+    typedef short i16x8 __attribute__((ext_vector_type(8)));
+    i16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(V8, v);
+}
+
+// ---- global access ------------------------------------------------------------------------
+__device__ __forceinline__ i32x4 gld16(const void* p) { return *reinterpret_cast<const i32x4*>(p); }
+__device__ __forceinline__ void gst16(void* p, i32x4 v) { *reinterpret_cast<i32x4*>(p) = v; }
+
+template <typename T> __device__ __forceinline__ float to_f32(T x) { return (float)x; }
+
+// bias element -> fp32 (natural units); E is the storage type selected by the bias kind
+template <int BIAS> struct BiasElem;
+template <> struct BiasElem<0> { typedef unsigned char type; };
+template <> struct BiasElem<1> { typedef unsigned char type; };
+template <> struct BiasElem<2> { typedef _Float16 type; };
+template <> struct BiasElem<3> { typedef __bf16 type; };
+template <> struct BiasElem<4> { typedef float type; };
+
+// Work-group id -> (tile, batch*head).  Work-groups are dealt round-robin to the 8 XCDs; when
+// the number of (batch, head) pairs is a multiple of 8 every tile of one pair is sent to the same
+// XCD so that its K/V (or Q/dO) stay in that XCD's L2.
+__device__ __forceinline__ void decode_block(int id, int n_tiles, int BH, int& tile, int& bh) {
+    if ((BH & 7) == 0) {
+        int xcd = id & 7, slot = id >> 3;
+        bh = (slot / n_tiles) * 8 + xcd;
+        tile = slot % n_tiles;
+    } else {
+        bh = id / n_tiles;
+        tile = id % n_tiles;
+    }
+}
+
+}  // namespace fa

@@ -1,0 +1,52 @@
+// Kernel argument blocks (host fills them from the C-ABI structs after validation).
+#pragma once
+#include <stdint.h>
+
+namespace fa {
+
+// strides in elements; index 0 = batch, 1 = sequence, 2 = head (the head-dim stride is 1)
+struct Strides3 {
+    int64_t b, s, h;
+};
+// bias / dbias: (B, H, M, N), any strides
+struct Strides4 {
+    int64_t b, h, m, n;
+};
+
+struct FwdParams {
+    const void* q;
+    const void* k;
+    const void* v;
+    const void* bias;
+    void* o;
+    float* lse;  // (B, H, M)
+    Strides3 sq, sk, sv, so;
+    Strides4 sbias;
+    int B, H, M, N;
+    float sm_scale;
+    int bias_vec;  // bias rows may be read with aligned 16-byte loads
+    int n_mtiles;
+};
+
+struct BwdParams {
+    const void* q;
+    const void* k;
+    const void* v;
+    const void* o;
+    const void* dout;
+    const void* bias;
+    const float* lse;  // (B, H, M)
+    float* delta;      // (B, H, M)        workspace
+    float* dq_acc;     // (B, H, M, D) fp32 workspace, zero on entry of the main kernel
+    void* dq;
+    void* dk;
+    void* dv;
+    void* dbias;
+    Strides3 sq, sk, sv, so, sdo, sdq, sdk, sdv;
+    Strides4 sbias, sdbias;
+    int B, H, M, N;
+    float sm_scale;
+    int n_ntiles;
+};
+
+}  // namespace fa

@@ -1,6 +1,461 @@
+// Backward attention kernels for gfx950: dQ, dK, dV and dBias in a single pass over the score
+// matrix (5 matrix products per tile, bias read once, dBias written once).
+//
+// Replaces _attn_bwd_preprocess, _attn_bwd_dkdv and _attn_bwd_dq of the reference
+// (/root/reference/flash_attention.py:197-646) and the host-side K / bias pre-scales
+// (flash_attention.py:699-704), which become fp32 multiplies inside the kernel.
+//
+//   fa_bwd_prep_kernel     delta[b,h,m] = sum_d o * do  (flash_attention.py:215-227) and zero fill
+//                          of the fp32 dQ accumulator
+//   fa_bwd_kernel          one work-group (4 waves) owns 128 keys of one (batch, head); wave w owns
+//                          32 of them with K and V held in registers as B operands.  Query rows
+//                          are streamed in blocks of 32 through LDS.  Per block:
+//                            S  = Q K^T, dP = dO V^T          (A = rows of Q / dO from LDS)
+//                            P  = 2^(S*scale + bias - LSE),  dS = P (dP - delta)
+//                            dV^T += dO^T P,  dK^T += Q^T dS  (A = columns of dO / Q gathered with
+//                                                              ds_read_b64_tr_b16, B = P / dS
+//                                                              straight from the accumulators)
+//                            dBias tile <- dS                  (flash_attention.py:307-308)
+//                            dS -> LDS, then dQ += dS K over all 128 keys, each wave one 32-wide
+//                            slice of the head dim, added to the fp32 accumulator with atomics
+//   fa_bwd_dq_kernel       dq = (T)(accumulator * sm_scale)   (flash_attention.py:644-646)
+//
+// In the accumulators a lane holds one key (column l%32) and 16 query rows, so bias loads and
+// dBias stores are contiguous across the lanes of a half-wave.
 #include "fa_common.hpp"
 #include "fa_params.hpp"
+
 namespace fa {
-hipError_t launch_bwd(const BwdParams&, int, int, int, bool, bool, hipStream_t) { return hipErrorNotSupported; }
-int bwd_block_n(int D) { return 128; }
+
+// Row-major LDS tile of 16-bit elements, D per row, no padding; 16-byte chunks are XOR-swizzled
+// by a function of the row so that both 16-byte row reads (lane = row) and 4-row column gathers
+// (ds_read_b64_tr_b16) are free of bank conflicts.
+template <int D> struct Swz {
+    static constexpr int CPR = D / 8;
+    __device__ static __forceinline__ int f(int row) {
+        if (CPR >= 16) return ((row & 3) << 2) | ((row >> 2) & 3);
+        if (CPR == 8) return (((row >> 1) & 1) << 2) | ((row >> 2) & 3);
+        if (CPR == 4) return (row >> 2) & 3;
+        return (row >> 3) & 1;
+    }
+    __device__ static __forceinline__ int off(int row, int col) {
+        return row * D + ((((col >> 3) ^ f(row)) << 3) | (col & 7));
+    }
+    // 8 k-slots gathered down column col0 + lane%32: rows row0 + 4g + {0..3}, row0 + 8 + 4g + {0..3}
+    template <typename V8, typename T>
+    __device__ static __forceinline__ V8 col8(const T* tile, int lane, int row0, int col0) {
+        const int g = lane >> 5, s = lane & 15;
+        const int row = row0 + 4 * g + (s >> 2);
+        const int col = (col0 + ((lane >> 4) & 1) * 16 + (s & 3) * 4) & (D - 1);
+        i16x4 lo = lds_read_tr4(tile + off(row, col));
+        i16x4 hi = lds_read_tr4(tile + off(row + 8, col));
+        typedef short i16x8 __attribute__((ext_vector_type(8)));
+        return __builtin_bit_cast(V8, (i16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    }
+};
+
+// ---------------------------------------------------------------------------------------------
+template <typename T, int D>
+__global__ __launch_bounds__(256) void fa_bwd_prep_kernel(const BwdParams p) {
+    constexpr int LPR = D / 8;         // lanes per row (16 bytes each)
+    constexpr int RPB = 256 / LPR;     // rows per block
+    typedef typename VecOf<T>::v8 T8;
+    const int64_t rows = (int64_t)p.B * p.H * p.M;
+    const int64_t row = (int64_t)blockIdx.x * RPB + threadIdx.x / LPR;
+    const int c = threadIdx.x % LPR;
+    float acc = 0.f;
+    if (row < rows) {
+        const int m = (int)(row % p.M);
+        const int bh = (int)(row / p.M);
+        const int b = bh / p.H, h = bh % p.H;
+        const T* op = reinterpret_cast<const T*>(p.o) + (int64_t)b * p.so.b + (int64_t)m * p.so.s + (int64_t)h * p.so.h;
+        const T* dp = reinterpret_cast<const T*>(p.dout) + (int64_t)b * p.sdo.b + (int64_t)m * p.sdo.s + (int64_t)h * p.sdo.h;
+        T8 ov = as_vec<T8>(gld16(op + c * 8));
+        T8 dv = as_vec<T8>(gld16(dp + c * 8));
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc += (float)ov[e] * (float)dv[e];
+        f32x4 z = {0.f, 0.f, 0.f, 0.f};
+        f32x4* za = reinterpret_cast<f32x4*>(p.dq_acc + row * D + c * 8);
+        za[0] = z;
+        za[1] = z;
+    }
+#pragma unroll
+    for (int w = LPR / 2; w >= 1; w >>= 1) acc += __shfl_xor(acc, w, 64);
+    if (row < rows && c == 0) p.delta[row] = acc;
 }
+
+template <typename T, int D>
+__global__ __launch_bounds__(256) void fa_bwd_dq_kernel(const BwdParams p) {
+    constexpr int LPR = D / 8;
+    constexpr int RPB = 256 / LPR;
+    typedef typename VecOf<T>::v8 T8;
+    const int64_t rows = (int64_t)p.B * p.H * p.M;
+    const int64_t row = (int64_t)blockIdx.x * RPB + threadIdx.x / LPR;
+    const int c = threadIdx.x % LPR;
+    if (row >= rows) return;
+    const int m = (int)(row % p.M);
+    const int bh = (int)(row / p.M);
+    const int b = bh / p.H, h = bh % p.H;
+    const f32x4* src = reinterpret_cast<const f32x4*>(p.dq_acc + row * D + c * 8);
+    f32x4 lo = src[0], hi = src[1];
+    T8 out;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        out[e] = (T)(lo[e] * p.sm_scale);
+        out[4 + e] = (T)(hi[e] * p.sm_scale);
+    }
+    T* dqp = reinterpret_cast<T*>(p.dq) + (int64_t)b * p.sdq.b + (int64_t)m * p.sdq.s + (int64_t)h * p.sdq.h;
+    gst16(dqp + c * 8, as_raw(out));
+}
+
+// ---------------------------------------------------------------------------------------------
+template <int D> struct BwdCfg {
+    static constexpr int BN = 128, BMI = 32, NT = 256;
+    static constexpr int DP = D < 32 ? 32 : D;
+    static constexpr int DB = DP / 32;
+    static constexpr int KSTEPS = D / 16;
+    static constexpr int CPR = D / 8;
+    static constexpr int NCH = (BMI * CPR + NT - 1) / NT;  // 16-byte chunks per thread per Q (or dO) block
+    static constexpr int DSS = BN + 8;                     // dS tile row stride (elements)
+    static constexpr int KTS = DP + 32;                    // one-time K tile (column gathers) row stride
+    static constexpr int Q_BYTES = BMI * D * 2;
+    static constexpr int DS_BYTES = BMI * DSS * 2;
+    static constexpr int STAT_BYTES = 2 * BMI * 4;
+    static constexpr int LOOP_BYTES = 2 * Q_BYTES + DS_BYTES + STAT_BYTES;
+    static constexpr int KT_BYTES = BN * KTS * 2;
+    static constexpr int LDS_BYTES = LOOP_BYTES > KT_BYTES ? LOOP_BYTES : KT_BYTES;
+    static constexpr int DQ_BLOCKS = DB;                   // 32 x 32 blocks of dQ per query block
+};
+
+template <typename T, int D, int BIAS, bool CAUSAL, bool DBIAS>
+__global__ __launch_bounds__(256, 1) void fa_bwd_kernel(const BwdParams p) {
+    typedef BwdCfg<D> C;
+    typedef Swz<D> SW;
+    typedef typename VecOf<T>::v8 T8;
+    typedef typename VecOf<T>::v4 T4;
+    typedef typename BiasElem<BIAS>::type E;
+    constexpr int BN = C::BN, BMI = C::BMI, CPR = C::CPR, DSS = C::DSS;
+
+    __shared__ __align__(16) unsigned char smem[C::LDS_BYTES];
+    T* q_lds = reinterpret_cast<T*>(smem);
+    T* do_lds = reinterpret_cast<T*>(smem + C::Q_BYTES);
+    T* ds_lds = reinterpret_cast<T*>(smem + 2 * C::Q_BYTES);
+    float* lse_lds = reinterpret_cast<float*>(smem + 2 * C::Q_BYTES + C::DS_BYTES);
+    float* delta_lds = lse_lds + BMI;
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int r = lane & 31, g = lane >> 5;
+
+    int nt, bh;
+    decode_block(blockIdx.x, p.n_ntiles, p.B * p.H, nt, bh);
+    const int b = bh / p.H, h = bh % p.H;
+    const int M = p.M, N = p.N;
+    const int n0 = nt * BN;
+    const int nw = n0 + wave * 32;
+    const int my_n = nw + r;
+
+    const T* qp = reinterpret_cast<const T*>(p.q) + (int64_t)b * p.sq.b + (int64_t)h * p.sq.h;
+    const T* kp = reinterpret_cast<const T*>(p.k) + (int64_t)b * p.sk.b + (int64_t)h * p.sk.h;
+    const T* vp = reinterpret_cast<const T*>(p.v) + (int64_t)b * p.sv.b + (int64_t)h * p.sv.h;
+    const T* dop = reinterpret_cast<const T*>(p.dout) + (int64_t)b * p.sdo.b + (int64_t)h * p.sdo.h;
+    const float* lsep = p.lse + ((int64_t)b * p.H + h) * M;
+    const float* deltap = p.delta + ((int64_t)b * p.H + h) * M;
+    float* dqap = p.dq_acc + ((int64_t)b * p.H + h) * M * D;
+    const E* bp = nullptr;
+    E* dbp = nullptr;
+    if (BIAS != 0) bp = reinterpret_cast<const E*>(p.bias) + (int64_t)b * p.sbias.b + (int64_t)h * p.sbias.h;
+    if (DBIAS) dbp = reinterpret_cast<E*>(p.dbias) + (int64_t)b * p.sdbias.b + (int64_t)h * p.sdbias.h;
+
+    // ---- K and V of this wave's 32 keys as B operands (column my_n, k = d) ----
+    T8 kreg[C::KSTEPS], vreg[C::KSTEPS];
+#pragma unroll
+    for (int ks = 0; ks < C::KSTEPS; ks++) {
+        i32x4 kr = {0, 0, 0, 0}, vr = {0, 0, 0, 0};
+        if (my_n < N) {
+            kr = gld16(kp + (int64_t)my_n * p.sk.s + ks * 16 + 8 * g);
+            vr = gld16(vp + (int64_t)my_n * p.sv.s + ks * 16 + 8 * g);
+        }
+        kreg[ks] = as_vec<T8>(kr);
+        vreg[ks] = as_vec<T8>(vr);
+    }
+
+    // ---- K of all 128 keys as B operand of dQ = dS K: column d = 32*dq_db + l%32, k = key.
+    // Staged once through LDS and gathered down the columns.  Wave w computes head-dim block
+    // dq_db of query sub-block 0 (blocks are dealt to waves round-robin; BMI = 32 has one
+    // sub-block, so only the first DQ_BLOCKS waves take part).
+    const int dq_db = wave % C::DQ_BLOCKS;
+    const bool dq_active = wave < C::DQ_BLOCKS;
+    T8 ktreg[BN / 16];
+    {
+        T* kt_lds = reinterpret_cast<T*>(smem);
+        for (int c = tid; c < BN * CPR; c += C::NT) {
+            int row = c / CPR, ch = c % CPR;
+            i32x4 v = {0, 0, 0, 0};
+            if (n0 + row < N) v = gld16(kp + (int64_t)(n0 + row) * p.sk.s + ch * 8);
+            lds_write16(kt_lds + row * C::KTS + ch * 8, v);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int ks = 0; ks < BN / 16; ks++) {
+            // natural key order in the k slots: rows 16 ks + 8 g + {0..7}
+            const int s = lane & 15;
+            const int col = (dq_db * 32 + ((lane >> 4) & 1) * 16 + (s & 3) * 4) & (D - 1);
+            const int row = ks * 16 + 8 * g + (s >> 2);
+            i16x4 lo = lds_read_tr4(kt_lds + row * C::KTS + col);
+            i16x4 hi = lds_read_tr4(kt_lds + (row + 4) * C::KTS + col);
+            typedef short i16x8 __attribute__((ext_vector_type(8)));
+            ktreg[ks] = __builtin_bit_cast(T8, (i16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        }
+        // the loop's first barrier separates these reads from the first tile writes
+    }
+
+    f32x16 dv_acc[C::DB], dk_acc[C::DB];
+#pragma unroll
+    for (int db = 0; db < C::DB; db++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            dv_acc[db][i] = 0.f;
+            dk_acc[db][i] = 0.f;
+        }
+
+    const float qk_scale = p.sm_scale * kLog2e;
+    const int n_mblocks = (M + BMI - 1) / BMI;
+    // causal: query blocks that end above the first key of this tile see none of its keys
+    const int mb_first = CAUSAL ? (n0 / BMI) : 0;
+
+    // blocks skipped by the causal schedule still owe zeros to dBias
+    if (DBIAS && CAUSAL) {
+        for (int mb = 0; mb < mb_first && mb < n_mblocks; mb++) {
+#pragma unroll 1
+            for (int i = 0; i < 16; i++) {
+                const int m = mb * BMI + 8 * (i >> 2) + 4 * g + (i & 3);
+                if (m < M && my_n < N) dbp[(int64_t)m * p.sdbias.m + (int64_t)my_n * p.sdbias.n] = (E)0.f;
+            }
+        }
+    }
+
+    i32x4 qreg[C::NCH], doreg[C::NCH];
+    float lse_r = 0.f, delta_r = 0.f;
+    auto prefetch = [&](int mb) {
+        const int m0 = mb * BMI;
+#pragma unroll
+        for (int it = 0; it < C::NCH; it++) {
+            int c = it * C::NT + tid;
+            int row = c / CPR, ch = c % CPR;
+            bool ok = (c < BMI * CPR) && (m0 + row < M);
+            i32x4 z = {0, 0, 0, 0};
+            qreg[it] = ok ? gld16(qp + (int64_t)(m0 + row) * p.sq.s + ch * 8) : z;
+            doreg[it] = ok ? gld16(dop + (int64_t)(m0 + row) * p.sdo.s + ch * 8) : z;
+        }
+        if (tid < BMI) {
+            lse_r = (m0 + tid < M) ? lsep[m0 + tid] : 0.f;
+            delta_r = (m0 + tid < M) ? deltap[m0 + tid] : 0.f;
+        }
+    };
+
+    if (mb_first < n_mblocks) prefetch(mb_first);
+
+    for (int mb = mb_first; mb < n_mblocks; mb++) {
+        const int m0 = mb * BMI;
+        __syncthreads();  // previous block fully consumed (Q/dO tiles and the dS tile)
+#pragma unroll
+        for (int it = 0; it < C::NCH; it++) {
+            int c = it * C::NT + tid;
+            int row = c / CPR, ch = c % CPR;
+            if (c < BMI * CPR) {
+                lds_write16(q_lds + SW::off(row, ch * 8), qreg[it]);
+                lds_write16(do_lds + SW::off(row, ch * 8), doreg[it]);
+            }
+        }
+        if (tid < BMI) {
+            lse_lds[tid] = lse_r;
+            delta_lds[tid] = delta_r;
+        }
+        __syncthreads();
+        if (mb + 1 < n_mblocks) prefetch(mb + 1);
+
+        const bool need_mask = (m0 + BMI > M) || (n0 + BN > N) || (CAUSAL && m0 < n0 + BN - 1);
+
+        // ---- bias for this wave's 32 x 32 block, accumulator layout: register i = row
+        // m0 + 8 (i/4) + 4 g + i%4, lanes of a half-wave = 32 consecutive keys ----
+        float bv[16];
+        if (BIAS != 0) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int m = m0 + 8 * (i >> 2) + 4 * g + (i & 3);
+                bv[i] = 0.f;
+                if (m < M && my_n < N) {
+                    E raw = bp[(int64_t)m * p.sbias.m + (int64_t)my_n * p.sbias.n];
+                    if constexpr (BIAS == 1) bv[i] = raw ? 0.f : kMask;
+                    else bv[i] = (float)raw * kLog2e;
+                } else if (BIAS != 0) {
+                    bv[i] = kMask;
+                }
+            }
+        }
+
+        // ---- S = Q K^T and dP = dO V^T ----
+        f32x16 s, dp;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            s[i] = 0.f;
+            dp[i] = 0.f;
+        }
+#pragma unroll
+        for (int ks = 0; ks < C::KSTEPS; ks++) {
+            T8 a = as_vec<T8>(lds_read16(q_lds + SW::off(r, ks * 16 + 8 * g)));
+            s = mfma32(a, kreg[ks], s);
+        }
+#pragma unroll
+        for (int ks = 0; ks < C::KSTEPS; ks++) {
+            T8 a = as_vec<T8>(lds_read16(do_lds + SW::off(r, ks * 16 + 8 * g)));
+            dp = mfma32(a, vreg[ks], dp);
+        }
+
+        // ---- P and dS (flash_attention.py:281-306) ----
+        T8 pT[2], dsT[2];
+#pragma unroll
+        for (int q4 = 0; q4 < 4; q4++) {
+            const f32x4 lse4 = *reinterpret_cast<const f32x4*>(lse_lds + 8 * q4 + 4 * g);
+            const f32x4 del4 = *reinterpret_cast<const f32x4*>(delta_lds + 8 * q4 + 4 * g);
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int i = q4 * 4 + e;
+                const int ml = 8 * q4 + 4 * g + e;  // row within the block
+                float x = __fmul_rn(s[i], qk_scale);
+                float add = (BIAS != 0) ? bv[i] : 0.f;
+                if (need_mask) {
+                    const int m = m0 + ml;
+                    float t = 0.f;
+                    if (m >= M || my_n >= N) t = kMask;
+                    if (CAUSAL && m < my_n) t += kMask;
+                    add = t + add;
+                }
+                x = __fadd_rn(x, add);
+                const float pv = fast_exp2(x - lse4[e]);
+                const float dsv = pv * (dp[i] - del4[e]);
+                pT[i >> 3][i & 7] = (T)pv;
+                dsT[i >> 3][i & 7] = (T)dsv;
+                ds_lds[ml * DSS + wave * 32 + r] = (T)dsv;
+                if (DBIAS) {
+                    const int m = m0 + ml;
+                    if (m < M && my_n < N) dbp[(int64_t)m * p.sdbias.m + (int64_t)my_n * p.sdbias.n] = (E)dsv;
+                }
+            }
+        }
+
+        // ---- dV^T += dO^T P and dK^T += Q^T dS ----
+#pragma unroll
+        for (int kk = 0; kk < 2; kk++) {
+#pragma unroll
+            for (int db = 0; db < C::DB; db++) {
+                T8 a = SW::template col8<T8>(do_lds, lane, kk * 16, db * 32);
+                dv_acc[db] = mfma32(a, pT[kk], dv_acc[db]);
+            }
+#pragma unroll
+            for (int db = 0; db < C::DB; db++) {
+                T8 a = SW::template col8<T8>(q_lds, lane, kk * 16, db * 32);
+                dk_acc[db] = mfma32(a, dsT[kk], dk_acc[db]);
+            }
+        }
+
+        __syncthreads();  // the dS tile of all 128 keys is complete
+
+        // ---- dQ block (32 rows x 32 head-dim columns) += dS K ----
+        if (dq_active) {
+            f32x16 dq;
+#pragma unroll
+            for (int i = 0; i < 16; i++) dq[i] = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < BN / 16; ks++) {
+                T8 a = as_vec<T8>(lds_read16(ds_lds + r * DSS + ks * 16 + 8 * g));
+                dq = mfma32(a, ktreg[ks], dq);
+            }
+            const int d = dq_db * 32 + r;
+            if (d < D) {
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    const int m = m0 + 8 * (i >> 2) + 4 * g + (i & 3);
+                    if (m < M)
+                        __hip_atomic_fetch_add(dqap + (int64_t)m * D + d, dq[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+        }
+    }
+
+    // ---- dK, dV of this wave's 32 keys (flash_attention.py:449-454) ----
+    if (my_n < N) {
+        T* dkp = reinterpret_cast<T*>(p.dk) + (int64_t)b * p.sdk.b + (int64_t)h * p.sdk.h + (int64_t)my_n * p.sdk.s;
+        T* dvp = reinterpret_cast<T*>(p.dv) + (int64_t)b * p.sdv.b + (int64_t)h * p.sdv.h + (int64_t)my_n * p.sdv.s;
+#pragma unroll
+        for (int db = 0; db < C::DB; db++) {
+#pragma unroll
+            for (int q4 = 0; q4 < 4; q4++) {
+                const int d = db * 32 + 8 * q4 + 4 * g;
+                if (d < D) {
+                    T4 kk4, vv4;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        kk4[e] = (T)(dk_acc[db][q4 * 4 + e] * p.sm_scale);
+                        vv4[e] = (T)dv_acc[db][q4 * 4 + e];
+                    }
+                    *reinterpret_cast<T4*>(dkp + d) = kk4;
+                    *reinterpret_cast<T4*>(dvp + d) = vv4;
+                }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+template <typename T, int D, int BIAS, bool CAUSAL, bool DBIAS>
+static hipError_t launch_main(const BwdParams& p, hipStream_t st) {
+    dim3 grid((unsigned)(p.n_ntiles * p.B * p.H));
+    hipLaunchKernelGGL((fa_bwd_kernel<T, D, BIAS, CAUSAL, DBIAS>), grid, dim3(256), 0, st, p);
+    return hipGetLastError();
+}
+
+template <typename T, int D> static hipError_t launch_all(const BwdParams& p, int bias, bool causal, bool dbias, hipStream_t st) {
+    constexpr int RPB = 256 / (D / 8);
+    const int64_t rows = (int64_t)p.B * p.H * p.M;
+    dim3 rgrid((unsigned)((rows + RPB - 1) / RPB));
+    hipLaunchKernelGGL((fa_bwd_prep_kernel<T, D>), rgrid, dim3(256), 0, st, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+#define FA_CASE(BK, DBK)                                                                                      \
+    if (bias == BK && dbias == DBK)                                                                           \
+        e = causal ? launch_main<T, D, BK, true, DBK>(p, st) : launch_main<T, D, BK, false, DBK>(p, st);
+    FA_CASE(0, false)
+    else FA_CASE(1, false)
+    else FA_CASE(2, false)
+    else FA_CASE(2, true)
+    else FA_CASE(3, false)
+    else FA_CASE(3, true)
+    else FA_CASE(4, false)
+    else FA_CASE(4, true)
+    else return hipErrorInvalidValue;
+#undef FA_CASE
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D>), rgrid, dim3(256), 0, st, p);
+    return hipGetLastError();
+}
+
+template <typename T> static hipError_t launch_d(const BwdParams& p, int D, int bias, bool causal, bool dbias, hipStream_t st) {
+    switch (D) {
+        case 16: return launch_all<T, 16>(p, bias, causal, dbias, st);
+        case 32: return launch_all<T, 32>(p, bias, causal, dbias, st);
+        case 64: return launch_all<T, 64>(p, bias, causal, dbias, st);
+        case 128: return launch_all<T, 128>(p, bias, causal, dbias, st);
+    }
+    return hipErrorNotSupported;
+}
+
+hipError_t launch_bwd(const BwdParams& p, int D, int dtype, int bias, bool causal, bool dbias, hipStream_t st) {
+    if (dtype == 0) return launch_d<_Float16>(p, D, bias, causal, dbias, st);
+    return launch_d<__bf16>(p, D, bias, causal, dbias, st);
+}
+
+int bwd_block_n(int D) { return D <= 128 ? 128 : 0; }
+
+}  // namespace fa

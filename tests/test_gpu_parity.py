@@ -1,0 +1,300 @@
+"""GPU parity tests: the HIP kernels, called through the C ABI (ctypes) by the public functions,
+against the fp32 oracle on the same seeded inputs.
+
+Tolerances (bf16 / fp16 inputs, fp32 oracle):  max-abs error <= 2e-2 on out;
+relative L2 error <= 5e-2 on each of dq, dk, dv, dbias;  masked keys contribute exactly zero.
+"""
+import math
+
+import pytest
+import torch
+
+import triton_flashattn_amd.flash_attention as fa_mod
+from triton_flashattn_amd import _native, flash_attention_fn, flash_attention_qkvpacked_fn
+from triton_flashattn_amd.flash_attention import _flash_attn_fwd
+from golden_io import golden_files, load_golden
+from oracle.attention_oracle import LN2, LOG2E, attention_backward, attention_forward
+
+pytestmark = pytest.mark.gpu
+
+OUT_ATOL = 2e-2
+GRAD_RTOL = 5e-2
+
+
+def rel_l2(a, b):
+    """||a - b|| / ||b||; a reference that is zero up to rounding (e.g. a softmax over a single
+    key has no gradient) is measured against an RMS floor of 1e-3 instead."""
+    b = b.float()
+    floor = 1e-3 * math.sqrt(b.numel())
+    return ((a.float() - b).norm() / b.norm().clamp_min(floor)).item()
+
+
+def make_inputs(dev, B, M, N, H, D, dtype, bias_kind, seed=0, trainable=True):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    mk = lambda *s: torch.randn(*s, generator=g).to(dtype).to(dev)
+    q, k, v, do = mk(B, M, H, D), mk(B, N, H, D), mk(B, N, H, D), mk(B, M, H, D)
+    bias = None
+    if bias_kind == "bool":
+        bias = (torch.rand(B, H, M, N, generator=g) > 0.3)
+        bias[..., 0] = True
+        bias = bias.to(dev)
+    elif bias_kind is not None:
+        bdt = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}[bias_kind]
+        bias = torch.randn(B, H, M, N, generator=g).to(bdt).to(dev)
+        if trainable:
+            bias.requires_grad_(True)
+    return q, k, v, do, bias
+
+
+def run_ours(q, k, v, do, bias, causal, sm_scale=None):
+    q, k, v = (t.detach().clone().requires_grad_(True) for t in (q, k, v))
+    out = flash_attention_fn(q, k, v, bias, causal, sm_scale)
+    out.backward(do)
+    res = {"out": out.detach(), "dq": q.grad, "dk": k.grad, "dv": v.grad, "dbias": None}
+    if bias is not None and bias.requires_grad:
+        res["dbias"] = bias.grad
+        bias.grad = None
+    return res
+
+
+def run_oracle(q, k, v, do, bias, causal, sm_scale=None):
+    b = None if bias is None else bias.detach()
+    out, lse2 = attention_forward(q, k, v, b, causal, sm_scale)
+    dq, dk, dv, dbias, _ = attention_backward(do, q, k, v, out, lse2, b, causal, sm_scale)
+    return {"out": out, "dq": dq, "dk": dk, "dv": dv, "dbias": dbias, "lse2": lse2}
+
+
+def check(ours, ref, tag=""):
+    err = (ours["out"].float() - ref["out"]).abs().max().item()
+    assert err <= OUT_ATOL, "%s out max-abs %.4g" % (tag, err)
+    for n in ("dq", "dk", "dv", "dbias"):
+        if ours[n] is not None:
+            e = rel_l2(ours[n], ref[n])
+            assert e <= GRAD_RTOL, "%s %s rel-L2 %.4g" % (tag, n, e)
+
+
+def test_hip_library_is_the_backend(gpu_device):
+    assert fa_mod._backend.name == "hip"
+    lib = _native.load()
+    assert lib.fa_abi_version() == _native.ABI_VERSION
+
+
+SHAPES = [  # B, M, N, H
+    (2, 128, 128, 2), (1, 256, 320, 3), (1, 100, 77, 2), (1, 1, 1, 1), (1, 129, 257, 1), (1, 33, 500, 2),
+]
+
+
+@pytest.mark.parametrize("D", [16, 32, 64, 128])
+@pytest.mark.parametrize("bias_kind", [None, "bool", "bf16", "f16", "f32"])
+def test_parity_noncausal(gpu_device, D, bias_kind):
+    for i, (B, M, N, H) in enumerate(SHAPES):
+        dtype = torch.bfloat16 if i % 2 == 0 else torch.float16
+        q, k, v, do, bias = make_inputs(gpu_device, B, M, N, H, D, dtype, bias_kind, seed=10 * D + i)
+        check(run_ours(q, k, v, do, bias, False), run_oracle(q, k, v, do, bias, False), "D%d %s %s" % (D, bias_kind, (B, M, N, H)))
+
+
+@pytest.mark.parametrize("D", [16, 32, 64, 128])
+@pytest.mark.parametrize("bias_kind", [None, "bool", "bf16", "f32"])
+def test_parity_causal(gpu_device, D, bias_kind):
+    for i, (B, S, H) in enumerate([(2, 256, 2), (1, 200, 2), (1, 129, 1), (1, 1, 1), (1, 513, 2)]):
+        dtype = torch.float16 if i % 2 == 0 else torch.bfloat16
+        q, k, v, do, bias = make_inputs(gpu_device, B, S, S, H, D, dtype, bias_kind, seed=7 * D + i)
+        check(run_ours(q, k, v, do, bias, True), run_oracle(q, k, v, do, bias, True), "D%d %s S%d" % (D, bias_kind, S))
+
+
+def test_forward_head_dim_256(gpu_device):
+    for causal, bias_kind in ((False, None), (True, "bf16"), (False, "bool")):
+        q, k, v, do, bias = make_inputs(gpu_device, 1, 200, 200, 2, 256, torch.bfloat16, bias_kind, trainable=False)
+        with torch.no_grad():
+            out = flash_attention_fn(q, k, v, bias, causal)
+        ref = run_oracle(q, k, v, do, bias, causal)
+        assert (out.float() - ref["out"]).abs().max().item() <= OUT_ATOL
+
+
+def test_sm_scale_and_untrainable_bias(gpu_device):
+    q, k, v, do, bias = make_inputs(gpu_device, 1, 150, 90, 2, 64, torch.bfloat16, "bf16", trainable=False)
+    ours = run_ours(q, k, v, do, bias, False, 0.05)
+    assert ours["dbias"] is None
+    check(ours, run_oracle(q, k, v, do, bias, False, 0.05))
+
+
+def test_lse_is_log2_sum_exp(gpu_device):
+    q, k, v, do, bias = make_inputs(gpu_device, 2, 300, 170, 3, 128, torch.bfloat16, "f32", trainable=False)
+    o, lse = _flash_attn_fwd(q, k, v, bias, False, 0.1)
+    s = torch.einsum("bmhd,bnhd->bhmn", q.float(), k.float()) * 0.1 + bias
+    assert lse.shape == (2, 3, 300)
+    assert torch.allclose(lse * LN2, torch.logsumexp(s, dim=-1), atol=2e-3, rtol=1e-4)
+
+
+def test_golden_fixtures(gpu_device):
+    for f in golden_files():
+        z = load_golden(f)
+        to = lambda t: None if t is None else t.to(gpu_device)
+        q, k, v, do = (to(z[n]).bfloat16() for n in ("q", "k", "v", "do"))
+        bias = to(z["bias"])
+        if bias is not None and bias.dtype != torch.bool:
+            bias = bias.bfloat16().requires_grad_(True)
+        ours = run_ours(q, k, v, do, bias, z["causal"], z["sm_scale"])
+        ref = {n: to(z[n]) for n in ("out", "dq", "dk", "dv", "dbias")}
+        check(ours, ref, f)
+
+
+# ---------------------------------------------------------------- BASELINE.json configs, full size
+def test_config1_cpu_reference_shape(gpu_device):
+    q, k, v, do, bias = make_inputs(gpu_device, 2, 128, 128, 4, 64, torch.bfloat16, "bf16", seed=0)
+    check(run_ours(q, k, v, do, bias, False), run_oracle(q, k, v, do, bias, False), "C1")
+
+
+def test_config2_causal_fp16(gpu_device):
+    q, k, v, do, _ = make_inputs(gpu_device, 4, 2048, 2048, 16, 64, torch.float16, None, seed=2)
+    check(run_ours(q, k, v, do, None, True), run_oracle(q, k, v, do, None, True), "C2")
+
+
+def test_config3_trainable_bias_headline(gpu_device):
+    B, M, N, H, D = 2, 4096, 4096, 16, 128
+    q, k, v, do, _ = make_inputs(gpu_device, B, M, N, H, D, torch.bfloat16, None, seed=3)
+    bias = torch.randn(B, H, M, N, device=gpu_device, generator=torch.Generator(device=gpu_device).manual_seed(3))
+    bias = bias.bfloat16().requires_grad_(True)
+    ours = run_ours(q, k, v, do, bias, False)
+    ref = run_oracle(q, k, v, do, bias, False)
+    check(ours, ref, "C3")
+    # size-independent properties on the kernel's own outputs
+    db = ours["dbias"].float()
+    assert db.sum(-1).abs().max().item() < 2e-2                          # rows of dBias sum to zero
+    scale = D ** -0.5
+    dq_from_dbias = torch.einsum("bhmn,bnhd->bmhd", db, k.float()) * scale
+    dk_from_dbias = torch.einsum("bhmn,bmhd->bnhd", db, q.float()) * scale
+    assert rel_l2(ours["dq"], dq_from_dbias) < GRAD_RTOL
+    assert rel_l2(ours["dk"], dk_from_dbias) < GRAD_RTOL
+    del ref, db, dq_from_dbias, dk_from_dbias
+    with torch.no_grad():
+        ones = flash_attention_fn(q, k, torch.ones_like(v), bias, False)
+    assert (ones.float() - 1).abs().max().item() < 1e-2                  # v == 1 -> out == 1
+
+
+def test_config4_packed_key_padding_causal(gpu_device):
+    B, S, H, D = 8, 1024, 12, 64
+    g = torch.Generator().manual_seed(4)
+    qkv = torch.randn(B, S, 3, H, D, generator=g).bfloat16().to(gpu_device)
+    do = torch.randn(B, S, H, D, generator=g).bfloat16().to(gpu_device)
+    lens = torch.randint(512, 1025, (B,), generator=g).to(gpu_device)
+    keep = torch.arange(S, device=gpu_device)[None, :] < lens[:, None]                  # (B, S)
+    expanded = keep[:, None, None, :].expand(B, H, S, S)                               # stride-0 view
+    results = []
+    for bias in (expanded.contiguous(), expanded):
+        x = qkv.clone().requires_grad_(True)
+        out = flash_attention_qkvpacked_fn(x, bias, True)
+        out.backward(do)
+        results.append((out.detach(), x.grad))
+    assert torch.equal(results[0][0], results[1][0])
+    assert torch.equal(results[0][1][:, :, 1:], results[1][1][:, :, 1:])
+    out, dqkv = results[0]
+    ref = run_oracle(qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], do, expanded, True)
+    check({"out": out, "dq": dqkv[:, :, 0], "dk": dqkv[:, :, 1], "dv": dqkv[:, :, 2], "dbias": None}, ref, "C4")
+    # keys masked for every query get exactly zero gradient
+    dead = ~keep                                                                        # (B, S)
+    assert (dqkv[:, :, 1][dead] == 0).all() and (dqkv[:, :, 2][dead] == 0).all()
+
+
+def test_config5_cross_attention_alibi(gpu_device):
+    B, H, M, N, D = 1, 32, 1024, 8192, 128
+    q, k, v, do, _ = make_inputs(gpu_device, B, M, N, H, D, torch.bfloat16, None, seed=5)
+    slopes = 2.0 ** (-8.0 * (torch.arange(H, device=gpu_device) + 1) / H)
+    i = torch.arange(M, device=gpu_device, dtype=torch.float32)[:, None]
+    j = torch.arange(N, device=gpu_device, dtype=torch.float32)[None, :]
+    bias = (-slopes[:, None, None] * (i * N / M - j).abs())[None].bfloat16().requires_grad_(True)
+    check(run_ours(q, k, v, do, bias, False), run_oracle(q, k, v, do, bias, False), "C5")
+
+
+# ---------------------------------------------------------------- exactness of masks
+def test_masked_keys_contribute_exactly_zero(gpu_device):
+    # one key tile (N <= 128): every output, dq included, has a single writer and is reproducible
+    B, M, N, H, D = 2, 200, 120, 2, 64
+    q, k, v, do, _ = make_inputs(gpu_device, B, M, N, H, D, torch.bfloat16, None, seed=21)
+    mask = torch.ones(B, H, M, N, dtype=torch.bool, device=gpu_device)
+    mask[..., 70:] = False
+    a = run_ours(q, k, v, do, mask, False)
+    k2, v2 = k.clone(), v.clone()
+    k2[:, 70:] = 3.0
+    v2[:, 70:] = -5.0
+    b = run_ours(q, k2, v2, do, mask, False)
+    for n in ("out", "dq"):
+        assert torch.equal(a[n], b[n]), n
+    assert torch.equal(a["dk"][:, :70], b["dk"][:, :70]) and torch.equal(a["dv"][:, :70], b["dv"][:, :70])
+    assert (a["dk"][:, 70:] == 0).all() and (a["dv"][:, 70:] == 0).all()
+    assert (b["dk"][:, 70:] == 0).all() and (b["dv"][:, 70:] == 0).all()
+    # several key tiles: out, dk, dv have single writers; dq is summed with atomics across key tiles
+    B, M, N, H, D = 1, 300, 700, 2, 128
+    q, k, v, do, _ = make_inputs(gpu_device, B, M, N, H, D, torch.float16, None, seed=22)
+    mask = (torch.rand(1, 1, 1, N, device=gpu_device) > 0.5).expand(B, H, M, N)
+    a = run_ours(q, k, v, do, mask, False)
+    dead = ~mask[0, 0, 0]
+    k2, v2 = k.clone(), v.clone()
+    k2[:, dead] = 2.0
+    v2[:, dead] = 9.0
+    b = run_ours(q, k2, v2, do, mask, False)
+    assert torch.equal(a["out"], b["out"])
+    assert torch.equal(a["dk"][:, ~dead], b["dk"][:, ~dead]) and torch.equal(a["dv"][:, ~dead], b["dv"][:, ~dead])
+    assert (a["dk"][:, dead] == 0).all() and (a["dv"][:, dead] == 0).all()
+    assert rel_l2(a["dq"], b["dq"]) < 1e-3
+
+
+def test_fully_masked_rows_are_finite_and_match_oracle(gpu_device):
+    B, M, N, H, D = 1, 70, 150, 2, 64
+    q, k, v, do, _ = make_inputs(gpu_device, B, M, N, H, D, torch.bfloat16, None, seed=23)
+    mask = torch.rand(B, H, M, N, device=gpu_device) > 0.3
+    mask[..., 0] = True
+    mask[:, :, 5, :] = False
+    mask[:, :, 69, :] = False
+    ours = run_ours(q, k, v, do, mask, False)
+    for n in ("out", "dq", "dk", "dv"):
+        assert torch.isfinite(ours[n]).all(), n
+    ref = run_oracle(q, k, v, do, mask, False)
+    check(ours, ref, "fully masked rows")
+    assert (ours["out"][:, 5].float() - ref["out"][:, 5]).abs().max().item() <= OUT_ATOL
+
+
+def test_causal_equals_lower_triangular_mask(gpu_device):
+    B, S, H, D = 1, 300, 2, 64
+    q, k, v, do, _ = make_inputs(gpu_device, B, S, S, H, D, torch.bfloat16, None, seed=24)
+    tri = torch.ones(S, S, dtype=torch.bool, device=gpu_device).tril().expand(B, H, S, S)
+    a = run_ours(q, k, v, do, None, True)
+    b = run_ours(q, k, v, do, tri, False)
+    assert torch.equal(a["out"], b["out"])
+    for n in ("dq", "dk", "dv"):
+        assert rel_l2(a[n], b[n]) < 1e-3
+
+
+# ---------------------------------------------------------------- layouts
+def test_packed_equals_unpacked_bit_for_bit(gpu_device):
+    B, S, H, D = 2, 128, 3, 64     # one key tile: dq has a single writer too
+    g = torch.Generator().manual_seed(31)
+    qkv = torch.randn(B, S, 3, H, D, generator=g).bfloat16().to(gpu_device).requires_grad_(True)
+    do = torch.randn(B, S, H, D, generator=g).bfloat16().to(gpu_device)
+    out = flash_attention_qkvpacked_fn(qkv, None, True)
+    out.backward(do)
+    un = run_ours(qkv.detach()[:, :, 0], qkv.detach()[:, :, 1], qkv.detach()[:, :, 2], do, None, True)
+    assert torch.equal(out, un["out"])
+    assert torch.equal(qkv.grad, torch.stack([un["dq"], un["dk"], un["dv"]], dim=2))
+
+
+def test_noncontiguous_inputs_and_upstream_grad(gpu_device):
+    B, M, N, H, D = 2, 90, 140, 2, 64
+    q, k, v, do, bias = make_inputs(gpu_device, B, M, N, H, D, torch.bfloat16, "bf16", seed=32)
+    qs = torch.randn(B, H, M, D, device=gpu_device).bfloat16().transpose(1, 2)            # head-major memory
+    ks = torch.randn(B, N, H, 2 * D, device=gpu_device).bfloat16()[..., ::2]              # head-dim stride 2
+    dos = do.transpose(1, 2).contiguous().transpose(1, 2)
+    bias_t = torch.randn(B, H, N, M, device=gpu_device).bfloat16().transpose(2, 3).requires_grad_(True)
+    ours = run_ours(qs, ks, v, dos, bias_t, False)
+    ref = run_oracle(qs, ks, v, dos, bias_t, False)
+    check(ours, ref, "strided")
+    assert ours["dbias"].shape == bias_t.shape
+
+
+def test_repeatability(gpu_device):
+    q, k, v, do, bias = make_inputs(gpu_device, 1, 512, 512, 4, 128, torch.bfloat16, "bf16", seed=33)
+    a = run_ours(q, k, v, do, bias, False)
+    b = run_ours(q, k, v, do, bias, False)
+    for n in ("out", "dk", "dv", "dbias"):
+        assert torch.equal(a[n], b[n]), n
+    assert rel_l2(a["dq"], b["dq"]) < 1e-3      # fp32 atomics: order-dependent rounding only

@@ -102,6 +102,20 @@ size_t fa_bwd_workspace_bytes(const fa_problem *p);
  * Replaces _flash_attn_bwd, flash_attention.py:688-763 (K and bias pre-scale :699-704 included). */
 int fa_bwd(const fa_bwd_args *args, void *stream);
 
+/* The three stages fa_bwd enqueues, in order.  fa_bwd(args, stream) is
+ * fa_bwd_stages(args, stream, FA_STAGE_ALL). */
+enum fa_bwd_stage {
+    FA_STAGE_PREP = 1, /* delta = rowsum(o * do) (flash_attention.py:197-233) + zero fill of the dQ accumulator */
+    FA_STAGE_MAIN = 2, /* dK, dV, dBias and the fp32 dQ accumulator (flash_attention.py:237-646) */
+    FA_STAGE_DQ = 4,   /* dq = accumulator * sm_scale in the output dtype (flash_attention.py:644-646) */
+    FA_STAGE_ALL = 7
+};
+
+/* Enqueue only the selected stages of the backward (same arguments and checks as fa_bwd).
+ * No counterpart in the reference: it exists so that a benchmark or profiler can bracket one
+ * stage with events; results are only meaningful after all three stages ran in order. */
+int fa_bwd_stages(const fa_bwd_args *args, void *stream, int stages);
+
 #ifdef __cplusplus
 }
 #endif

@@ -29,7 +29,7 @@ class OracleBackend:
         o.copy_(out.to(o.dtype))
         lse.copy_(lse2)
 
-    def bwd(self, do, q, k, v, o, bias, causal, sm_scale, lse, dq, dk, dv, dbias):
+    def bwd(self, do, q, k, v, o, bias, causal, sm_scale, lse, dq, dk, dv, dbias, stages=7, workspace=None):
         self.calls.append(("bwd", dq.stride(), dk.stride(), dv.stride()))
         gq, gk, gv, gb, _ = attention_backward(do, q, k, v, o, lse, bias, causal, sm_scale)
         dq.copy_(gq.to(dq.dtype))

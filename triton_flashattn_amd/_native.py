@@ -46,7 +46,8 @@ class FaBwdArgs(ctypes.Structure):
     ]
 
 
-EXPORTS = ("fa_abi_version", "fa_strerror", "fa_fwd", "fa_bwd_workspace_bytes", "fa_bwd")
+EXPORTS = ("fa_abi_version", "fa_strerror", "fa_fwd", "fa_bwd_workspace_bytes", "fa_bwd", "fa_bwd_stages")
+FA_STAGE_PREP, FA_STAGE_MAIN, FA_STAGE_DQ, FA_STAGE_ALL = 1, 2, 4, 7
 
 _lib = None
 
@@ -75,6 +76,8 @@ def load():
     lib.fa_bwd_workspace_bytes.argtypes = [ctypes.POINTER(FaProblem)]
     lib.fa_bwd.restype = ctypes.c_int
     lib.fa_bwd.argtypes = [ctypes.POINTER(FaBwdArgs), ctypes.c_void_p]
+    lib.fa_bwd_stages.restype = ctypes.c_int
+    lib.fa_bwd_stages.argtypes = [ctypes.POINTER(FaBwdArgs), ctypes.c_void_p, ctypes.c_int]
     if lib.fa_abi_version() != ABI_VERSION:
         raise NativeLibraryError("libfa_mi355.so has ABI %d, expected %d" % (lib.fa_abi_version(), ABI_VERSION))
     _lib = lib

@@ -7,7 +7,7 @@
 
 namespace fa {
 hipError_t launch_fwd(const FwdParams& p, int D, int dtype, int bias, bool causal, hipStream_t st);
-hipError_t launch_bwd(const BwdParams& p, int D, int dtype, int bias, bool causal, bool dbias, hipStream_t st);
+hipError_t launch_bwd(const BwdParams& p, int D, int dtype, int bias, bool causal, bool dbias, int stages, hipStream_t st);
 int fwd_block_m();
 int bwd_block_n(int D);
 }  // namespace fa
@@ -117,8 +117,9 @@ size_t fa_bwd_workspace_bytes(const fa_problem* p) {
     return align256(rows * sizeof(float)) + align256(rows * p->D * sizeof(float));
 }
 
-int fa_bwd(const fa_bwd_args* a, void* stream) {
+int fa_bwd_stages(const fa_bwd_args* a, void* stream, int stages) {
     if (!a) return FA_ERR_NULL;
+    if (stages <= 0 || (stages & ~FA_STAGE_ALL)) return FA_ERR_UNSUPPORTED;
     const fa_problem& p = a->p;
     int st = check_problem(p);
     if (st != FA_OK) return st;
@@ -149,10 +150,12 @@ int fa_bwd(const fa_bwd_args* a, void* stream) {
     int bn = fa::bwd_block_n(p.D);
     if (bn <= 0) return FA_ERR_UNSUPPORTED;
     k.n_ntiles = (p.N + bn - 1) / bn;
-    hipError_t e = fa::launch_bwd(k, p.D, p.dtype, p.bias_dtype, p.causal != 0, a->dbias != nullptr,
+    hipError_t e = fa::launch_bwd(k, p.D, p.dtype, p.bias_dtype, p.causal != 0, a->dbias != nullptr, stages,
                                   static_cast<hipStream_t>(stream));
     if (e == hipErrorNotSupported) return FA_ERR_UNSUPPORTED;
     return e == hipSuccess ? FA_OK : FA_ERR_LAUNCH;
 }
+
+int fa_bwd(const fa_bwd_args* a, void* stream) { return fa_bwd_stages(a, stream, FA_STAGE_ALL); }
 
 }  // extern "C"

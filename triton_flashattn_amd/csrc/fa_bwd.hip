@@ -416,13 +416,17 @@ static hipError_t launch_main(const BwdParams& p, hipStream_t st) {
     return hipGetLastError();
 }
 
-template <typename T, int D> static hipError_t launch_all(const BwdParams& p, int bias, bool causal, bool dbias, hipStream_t st) {
+template <typename T, int D> static hipError_t launch_all(const BwdParams& p, int bias, bool causal, bool dbias, int stages, hipStream_t st) {
     constexpr int RPB = 256 / (D / 8);
     const int64_t rows = (int64_t)p.B * p.H * p.M;
     dim3 rgrid((unsigned)((rows + RPB - 1) / RPB));
-    hipLaunchKernelGGL((fa_bwd_prep_kernel<T, D>), rgrid, dim3(256), 0, st, p);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return e;
+    hipError_t e = hipSuccess;
+    if (stages & 1) {
+        hipLaunchKernelGGL((fa_bwd_prep_kernel<T, D>), rgrid, dim3(256), 0, st, p);
+        e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    if (stages & 2) {
 #define FA_CASE(BK, DBK)                                                                                      \
     if (bias == BK && dbias == DBK)                                                                           \
         e = causal ? launch_main<T, D, BK, true, DBK>(p, st) : launch_main<T, D, BK, false, DBK>(p, st);
@@ -436,24 +440,28 @@ template <typename T, int D> static hipError_t launch_all(const BwdParams& p, in
     else FA_CASE(4, true)
     else return hipErrorInvalidValue;
 #undef FA_CASE
-    if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D>), rgrid, dim3(256), 0, st, p);
-    return hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    if (stages & 4) {
+        hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D>), rgrid, dim3(256), 0, st, p);
+        e = hipGetLastError();
+    }
+    return e;
 }
 
-template <typename T> static hipError_t launch_d(const BwdParams& p, int D, int bias, bool causal, bool dbias, hipStream_t st) {
+template <typename T> static hipError_t launch_d(const BwdParams& p, int D, int bias, bool causal, bool dbias, int stages, hipStream_t st) {
     switch (D) {
-        case 16: return launch_all<T, 16>(p, bias, causal, dbias, st);
-        case 32: return launch_all<T, 32>(p, bias, causal, dbias, st);
-        case 64: return launch_all<T, 64>(p, bias, causal, dbias, st);
-        case 128: return launch_all<T, 128>(p, bias, causal, dbias, st);
+        case 16: return launch_all<T, 16>(p, bias, causal, dbias, stages, st);
+        case 32: return launch_all<T, 32>(p, bias, causal, dbias, stages, st);
+        case 64: return launch_all<T, 64>(p, bias, causal, dbias, stages, st);
+        case 128: return launch_all<T, 128>(p, bias, causal, dbias, stages, st);
     }
     return hipErrorNotSupported;
 }
 
-hipError_t launch_bwd(const BwdParams& p, int D, int dtype, int bias, bool causal, bool dbias, hipStream_t st) {
-    if (dtype == 0) return launch_d<_Float16>(p, D, bias, causal, dbias, st);
-    return launch_d<__bf16>(p, D, bias, causal, dbias, st);
+hipError_t launch_bwd(const BwdParams& p, int D, int dtype, int bias, bool causal, bool dbias, int stages, hipStream_t st) {
+    if (dtype == 0) return launch_d<_Float16>(p, D, bias, causal, dbias, stages, st);
+    return launch_d<__bf16>(p, D, bias, causal, dbias, stages, st);
 }
 
 int bwd_block_n(int D) { return D <= 128 ? 128 : 0; }

@@ -88,15 +88,23 @@ class _HipBackend:
             stream = torch.cuda.current_stream(dev).cuda_stream
             _native.check(lib.fa_fwd(ctypes.byref(a), ctypes.c_void_p(stream)))
 
-    def bwd(self, do, q, k, v, o, bias, causal, sm_scale, lse, dq, dk, dv, dbias):
+    def bwd_workspace(self, q, k, bias, causal, sm_scale):
+        """Scratch tensor of the size fa_bwd_workspace_bytes() asks for (delta + fp32 dQ accumulator)."""
+        p = self._problem(q, k, bias, causal, sm_scale)
+        nbytes = int(_native.load().fa_bwd_workspace_bytes(ctypes.byref(p)))
+        if nbytes == 0:
+            raise _native.NativeLibraryError("libfa_mi355: problem rejected by fa_bwd_workspace_bytes")
+        return torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+
+    def bwd(self, do, q, k, v, o, bias, causal, sm_scale, lse, dq, dk, dv, dbias,
+            stages=_native.FA_STAGE_ALL, workspace=None):
         dev = self._require_gpu(do, q, k, v, o, bias, lse, dq, dk, dv, dbias)
         lib = _native.load()
         a = _native.FaBwdArgs()
         a.p = self._problem(q, k, bias, causal, sm_scale)
-        nbytes = int(lib.fa_bwd_workspace_bytes(ctypes.byref(a.p)))
-        if nbytes == 0:
-            raise _native.NativeLibraryError("libfa_mi355: problem rejected by fa_bwd_workspace_bytes")
-        workspace = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        if workspace is None:
+            workspace = self.bwd_workspace(q, k, bias, causal, sm_scale)
+        nbytes = workspace.numel()
         a.q, a.k, a.v, a.o, a.dout, a.lse = (q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
                                              do.data_ptr(), lse.data_ptr())
         a.dq, a.dk, a.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
@@ -112,7 +120,7 @@ class _HipBackend:
             a.dbias_strides = _strides4(dbias)
         with torch.cuda.device(dev):
             stream = torch.cuda.current_stream(dev).cuda_stream
-            _native.check(lib.fa_bwd(ctypes.byref(a), ctypes.c_void_p(stream)))
+            _native.check(lib.fa_bwd_stages(ctypes.byref(a), ctypes.c_void_p(stream), int(stages)))
             # the workspace is only touched by work already enqueued on this stream; the caching
             # allocator re-issues it to later work on the same stream only, so it may be dropped
 

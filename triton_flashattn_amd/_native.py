@@ -6,7 +6,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libfa_mi355.so")
+# FA_MI355_LIB points at another build of the same ABI (e.g. an instrumented one)
+LIB_PATH = os.environ.get("FA_MI355_LIB") or os.path.join(_HERE, "libfa_mi355.so")
 ABI_VERSION = 1
 
 FA_F16, FA_BF16 = 0, 1

@@ -143,8 +143,14 @@ int fa_bwd_stages(const fa_bwd_args* a, void* stream, int stages) {
     k.dq_acc = reinterpret_cast<float*>(static_cast<char*>(a->workspace) + align256(rows * sizeof(float)));
     k.sq = s3(a->q_strides); k.sk = s3(a->k_strides); k.sv = s3(a->v_strides); k.so = s3(a->o_strides);
     k.sdo = s3(a->do_strides); k.sdq = s3(a->dq_strides); k.sdk = s3(a->dk_strides); k.sdv = s3(a->dv_strides);
-    if (a->bias) k.sbias = s4(a->bias_strides);
-    if (a->dbias) k.sdbias = s4(a->dbias_strides);
+    if (a->bias) {
+        k.sbias = s4(a->bias_strides);
+        k.bias_vec = bias_vec_ok(a->bias, a->bias_strides, p) ? 1 : 0;
+    }
+    if (a->dbias) {
+        k.sdbias = s4(a->dbias_strides);
+        k.dbias_vec = bias_vec_ok(a->dbias, a->dbias_strides, p) ? 1 : 0;
+    }
     k.B = p.B; k.H = p.H; k.M = p.M; k.N = p.N;
     k.sm_scale = p.sm_scale;
     int bn = fa::bwd_block_n(p.D);

@@ -9,7 +9,8 @@
 //                          of the fp32 dQ accumulator
 //   fa_bwd_kernel          one work-group (4 waves) owns 128 keys of one (batch, head); wave w owns
 //                          32 of them with K and V held in registers as B operands.  Query rows
-//                          are streamed in blocks of 32 through LDS.  Per block:
+//                          are streamed in blocks of 64 (two 32-row sub-blocks) through
+//                          double-buffered LDS tiles.  Per sub-block:
 //                            S  = Q K^T, dP = dO V^T          (A = rows of Q / dO from LDS)
 //                            P  = 2^(S*scale + bias - LSE),  dS = P (dP - delta)
 //                            dV^T += dO^T P,  dK^T += Q^T dS  (A = columns of dO / Q gathered with
@@ -109,8 +110,8 @@ __global__ __launch_bounds__(256) void fa_bwd_dq_kernel(const BwdParams p) {
 }
 
 // ---------------------------------------------------------------------------------------------
-template <int D> struct BwdCfg {
-    static constexpr int BN = 128, BMI = 32, NT = 256;
+template <int D, int BIAS> struct BwdCfg {
+    static constexpr int BN = 128, BMI = 64, NSUB = BMI / 32, NT = 256;
     static constexpr int DP = D < 32 ? 32 : D;
     static constexpr int DB = DP / 32;
     static constexpr int KSTEPS = D / 16;
@@ -118,30 +119,37 @@ template <int D> struct BwdCfg {
     static constexpr int NCH = (BMI * CPR + NT - 1) / NT;  // 16-byte chunks per thread per Q (or dO) block
     static constexpr int DSS = BN + 8;                     // dS tile row stride (elements)
     static constexpr int KTS = DP + 32;                    // one-time K tile (column gathers) row stride
+    static constexpr int ES = BIAS == 0 ? 0 : (BIAS == 1 ? 1 : (BIAS == 4 ? 4 : 2));
+    static constexpr int BCH = (BMI * 32 * ES) / (64 * 16);  // 16-byte bias chunks per lane per block
+    static constexpr int BCPR = 2 * ES;                    // 16-byte chunks per 32-key bias row
     static constexpr int Q_BYTES = BMI * D * 2;
     static constexpr int DS_BYTES = BMI * DSS * 2;
     static constexpr int STAT_BYTES = 2 * BMI * 4;
-    static constexpr int LOOP_BYTES = 2 * Q_BYTES + DS_BYTES + STAT_BYTES;
+    static constexpr int BT_BYTES = BMI * 32 * ES;         // wave-private bias tile
+    static constexpr int OFF_DO = 2 * Q_BYTES;
+    static constexpr int OFF_DS = 4 * Q_BYTES;
+    static constexpr int OFF_STAT = OFF_DS + 2 * DS_BYTES;
+    static constexpr int OFF_BIAS = OFF_STAT + 2 * STAT_BYTES;
+    static constexpr int LOOP_BYTES = OFF_BIAS + 4 * BT_BYTES;
     static constexpr int KT_BYTES = BN * KTS * 2;
     static constexpr int LDS_BYTES = LOOP_BYTES > KT_BYTES ? LOOP_BYTES : KT_BYTES;
-    static constexpr int DQ_BLOCKS = DB;                   // 32 x 32 blocks of dQ per query block
+    static constexpr int NDQ = NSUB * DB;                  // 32 x 32 blocks of dQ per query block
+    static constexpr int BPW = NDQ >= 4 ? NDQ / 4 : 1;     // dQ blocks per wave
 };
 
 template <typename T, int D, int BIAS, bool CAUSAL, bool DBIAS>
 __global__ __launch_bounds__(256, 1) void fa_bwd_kernel(const BwdParams p) {
-    typedef BwdCfg<D> C;
+    typedef BwdCfg<D, BIAS> C;
     typedef Swz<D> SW;
     typedef typename VecOf<T>::v8 T8;
     typedef typename VecOf<T>::v4 T4;
     typedef typename BiasElem<BIAS>::type E;
-    constexpr int BN = C::BN, BMI = C::BMI, CPR = C::CPR, DSS = C::DSS;
+    constexpr int BN = C::BN, BMI = C::BMI, CPR = C::CPR, DSS = C::DSS, NSUB = C::NSUB;
+    // dBias leaves through the dS tile (16-byte row stores) when it has the element type of dS
+    constexpr bool DB_VIA_LDS = DBIAS && ((BIAS == 2 && sizeof(T) == 2 && __is_same(T, _Float16)) ||
+                                          (BIAS == 3 && __is_same(T, __bf16)));
 
     __shared__ __align__(16) unsigned char smem[C::LDS_BYTES];
-    T* q_lds = reinterpret_cast<T*>(smem);
-    T* do_lds = reinterpret_cast<T*>(smem + C::Q_BYTES);
-    T* ds_lds = reinterpret_cast<T*>(smem + 2 * C::Q_BYTES);
-    float* lse_lds = reinterpret_cast<float*>(smem + 2 * C::Q_BYTES + C::DS_BYTES);
-    float* delta_lds = lse_lds + BMI;
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
@@ -166,6 +174,7 @@ __global__ __launch_bounds__(256, 1) void fa_bwd_kernel(const BwdParams p) {
     E* dbp = nullptr;
     if (BIAS != 0) bp = reinterpret_cast<const E*>(p.bias) + (int64_t)b * p.sbias.b + (int64_t)h * p.sbias.h;
     if (DBIAS) dbp = reinterpret_cast<E*>(p.dbias) + (int64_t)b * p.sdbias.b + (int64_t)h * p.sdbias.h;
+    unsigned char* bt_lds = smem + C::OFF_BIAS + wave * C::BT_BYTES;
 
     // ---- K and V of this wave's 32 keys as B operands (column my_n, k = d) ----
     T8 kreg[C::KSTEPS], vreg[C::KSTEPS];
@@ -181,11 +190,13 @@ __global__ __launch_bounds__(256, 1) void fa_bwd_kernel(const BwdParams p) {
     }
 
     // ---- K of all 128 keys as B operand of dQ = dS K: column d = 32*dq_db + l%32, k = key.
-    // Staged once through LDS and gathered down the columns.  Wave w computes head-dim block
-    // dq_db of query sub-block 0 (blocks are dealt to waves round-robin; BMI = 32 has one
-    // sub-block, so only the first DQ_BLOCKS waves take part).
-    const int dq_db = wave % C::DQ_BLOCKS;
-    const bool dq_active = wave < C::DQ_BLOCKS;
+    // Staged once through LDS and gathered down the columns.  The NDQ = NSUB * DB blocks of dQ of
+    // a query block are dealt to the waves: wave w owns blocks w*BPW .. w*BPW+BPW-1, block index
+    // = (head-dim block) * NSUB + (query sub-block), so all blocks of a wave share one head-dim
+    // block and therefore one set of K^T registers.
+    const int dq_first = wave * C::BPW;
+    const int dq_db = dq_first / NSUB;
+    const bool dq_active = dq_first < C::NDQ;
     T8 ktreg[BN / 16];
     {
         T* kt_lds = reinterpret_cast<T*>(smem);
@@ -200,14 +211,14 @@ __global__ __launch_bounds__(256, 1) void fa_bwd_kernel(const BwdParams p) {
         for (int ks = 0; ks < BN / 16; ks++) {
             // natural key order in the k slots: rows 16 ks + 8 g + {0..7}
             const int s = lane & 15;
-            const int col = (dq_db * 32 + ((lane >> 4) & 1) * 16 + (s & 3) * 4) & (D - 1);
+            const int col = ((dq_active ? dq_db : 0) * 32 + ((lane >> 4) & 1) * 16 + (s & 3) * 4) & (D - 1);
             const int row = ks * 16 + 8 * g + (s >> 2);
             i16x4 lo = lds_read_tr4(kt_lds + row * C::KTS + col);
             i16x4 hi = lds_read_tr4(kt_lds + (row + 4) * C::KTS + col);
             typedef short i16x8 __attribute__((ext_vector_type(8)));
             ktreg[ks] = __builtin_bit_cast(T8, (i16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
         }
-        // the loop's first barrier separates these reads from the first tile writes
+        __syncthreads();  // the staging area is reused by the loop's tiles
     }
 
     f32x16 dv_acc[C::DB], dk_acc[C::DB];
@@ -224,18 +235,29 @@ __global__ __launch_bounds__(256, 1) void fa_bwd_kernel(const BwdParams p) {
     // causal: query blocks that end above the first key of this tile see none of its keys
     const int mb_first = CAUSAL ? (n0 / BMI) : 0;
 
+    // 16-byte chunk (row, ch) of this wave's 32-key slice of a (B, H, M, N) bias-like tensor
+    const bool bias_vec = BIAS != 0 && p.bias_vec;
+    const bool dbias_vec = DBIAS && p.dbias_vec;
+    constexpr int EPC = C::ES > 0 ? 16 / C::ES : 8;  // elements per 16-byte chunk
+
     // blocks skipped by the causal schedule still owe zeros to dBias
     if (DBIAS && CAUSAL) {
-        for (int mb = 0; mb < mb_first && mb < n_mblocks; mb++) {
-#pragma unroll 1
-            for (int i = 0; i < 16; i++) {
-                const int m = mb * BMI + 8 * (i >> 2) + 4 * g + (i & 3);
-                if (m < M && my_n < N) dbp[(int64_t)m * p.sdbias.m + (int64_t)my_n * p.sdbias.n] = (E)0.f;
+        const int rows_skipped = mb_first * BMI < M ? mb_first * BMI : M;
+        for (int c = lane; c < rows_skipped * C::BCPR; c += 64) {
+            const int m = c / C::BCPR, nn = nw + (c % C::BCPR) * EPC;
+            E* dst = dbp + (int64_t)m * p.sdbias.m + (int64_t)nn * p.sdbias.n;
+            if (dbias_vec && nn + EPC <= N) {
+                i32x4 z = {0, 0, 0, 0};
+                gst16(dst, z);
+            } else {
+                for (int e = 0; e < EPC; e++)
+                    if (nn + e < N) dst[(int64_t)e * p.sdbias.n] = (E)0.f;
             }
         }
     }
 
     i32x4 qreg[C::NCH], doreg[C::NCH];
+    i32x4 breg[C::BCH > 0 ? C::BCH : 1];
     float lse_r = 0.f, delta_r = 0.f;
     auto prefetch = [&](int mb) {
         const int m0 = mb * BMI;
@@ -252,13 +274,31 @@ __global__ __launch_bounds__(256, 1) void fa_bwd_kernel(const BwdParams p) {
             lse_r = (m0 + tid < M) ? lsep[m0 + tid] : 0.f;
             delta_r = (m0 + tid < M) ? deltap[m0 + tid] : 0.f;
         }
+        if constexpr (BIAS != 0) {
+#pragma unroll
+            for (int it = 0; it < C::BCH; it++) {
+                const int c = it * 64 + lane;
+                const int m = m0 + c / C::BCPR, nn = nw + (c % C::BCPR) * EPC;
+                const E* src = bp + (int64_t)m * p.sbias.m + (int64_t)nn * p.sbias.n;
+                i32x4 v = {0, 0, 0, 0};
+                if (m < M) {
+                    if (bias_vec && nn + EPC <= N) {
+                        v = gld16(src);
+                    } else {
+                        E tmp[EPC];
+#pragma unroll
+                        for (int e = 0; e < EPC; e++) tmp[e] = (nn + e < N) ? src[(int64_t)e * p.sbias.n] : (E)0.f;
+                        v = __builtin_bit_cast(i32x4, tmp);
+                    }
+                }
+                breg[it] = v;
+            }
+        }
     };
-
-    if (mb_first < n_mblocks) prefetch(mb_first);
-
-    for (int mb = mb_first; mb < n_mblocks; mb++) {
-        const int m0 = mb * BMI;
-        __syncthreads();  // previous block fully consumed (Q/dO tiles and the dS tile)
+    auto stage = [&](int buf) {  // registers -> LDS tiles of buffer `buf`
+        T* q_lds = reinterpret_cast<T*>(smem + buf * C::Q_BYTES);
+        T* do_lds = reinterpret_cast<T*>(smem + C::OFF_DO + buf * C::Q_BYTES);
+        float* st = reinterpret_cast<float*>(smem + C::OFF_STAT + buf * C::STAT_BYTES);
 #pragma unroll
         for (int it = 0; it < C::NCH; it++) {
             int c = it * C::NT + tid;
@@ -269,116 +309,169 @@ __global__ __launch_bounds__(256, 1) void fa_bwd_kernel(const BwdParams p) {
             }
         }
         if (tid < BMI) {
-            lse_lds[tid] = lse_r;
-            delta_lds[tid] = delta_r;
+            st[tid] = lse_r;
+            st[BMI + tid] = delta_r;
         }
-        __syncthreads();
+    };
+
+    int buf = 0;
+    if (mb_first < n_mblocks) {
+        prefetch(mb_first);
+        stage(0);
+    }
+    __syncthreads();
+
+    for (int mb = mb_first; mb < n_mblocks; mb++, buf ^= 1) {
+        const int m0 = mb * BMI;
+        const T* q_lds = reinterpret_cast<const T*>(smem + buf * C::Q_BYTES);
+        const T* do_lds = reinterpret_cast<const T*>(smem + C::OFF_DO + buf * C::Q_BYTES);
+        T* ds_lds = reinterpret_cast<T*>(smem + C::OFF_DS + buf * C::DS_BYTES);
+        const float* lse_lds = reinterpret_cast<const float*>(smem + C::OFF_STAT + buf * C::STAT_BYTES);
+        const float* delta_lds = lse_lds + BMI;
+
+        // this block's bias slice: registers -> wave-private LDS tile [BMI][32]
+        if constexpr (BIAS != 0) {
+#pragma unroll
+            for (int it = 0; it < C::BCH; it++) lds_write16(bt_lds + (it * 64 + lane) * 16, breg[it]);
+        }
         if (mb + 1 < n_mblocks) prefetch(mb + 1);
 
         const bool need_mask = (m0 + BMI > M) || (n0 + BN > N) || (CAUSAL && m0 < n0 + BN - 1);
 
-        // ---- bias for this wave's 32 x 32 block, accumulator layout: register i = row
-        // m0 + 8 (i/4) + 4 g + i%4, lanes of a half-wave = 32 consecutive keys ----
-        float bv[16];
-        if (BIAS != 0) {
+        // ---- S = Q K^T and dP = dO V^T for both 32-row sub-blocks ----
+        f32x16 s[NSUB], dp[NSUB];
+#pragma unroll
+        for (int sb = 0; sb < NSUB; sb++) {
 #pragma unroll
             for (int i = 0; i < 16; i++) {
-                const int m = m0 + 8 * (i >> 2) + 4 * g + (i & 3);
-                bv[i] = 0.f;
-                if (m < M && my_n < N) {
-                    E raw = bp[(int64_t)m * p.sbias.m + (int64_t)my_n * p.sbias.n];
-                    if constexpr (BIAS == 1) bv[i] = raw ? 0.f : kMask;
-                    else bv[i] = (float)raw * kLog2e;
-                } else if (BIAS != 0) {
-                    bv[i] = kMask;
-                }
+                s[sb][i] = 0.f;
+                dp[sb][i] = 0.f;
+            }
+#pragma unroll
+            for (int ks = 0; ks < C::KSTEPS; ks++) {
+                T8 a = as_vec<T8>(lds_read16(q_lds + SW::off(sb * 32 + r, ks * 16 + 8 * g)));
+                s[sb] = mfma32(a, kreg[ks], s[sb]);
+            }
+#pragma unroll
+            for (int ks = 0; ks < C::KSTEPS; ks++) {
+                T8 a = as_vec<T8>(lds_read16(do_lds + SW::off(sb * 32 + r, ks * 16 + 8 * g)));
+                dp[sb] = mfma32(a, vreg[ks], dp[sb]);
             }
         }
 
-        // ---- S = Q K^T and dP = dO V^T ----
-        f32x16 s, dp;
+        // ---- P and dS (flash_attention.py:281-306); register i of sub-block sb is row
+        // m0 + 32 sb + 8 (i/4) + 4 g + i%4, the lane is key my_n ----
+        T8 pT[NSUB][2], dsT[NSUB][2];
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-            s[i] = 0.f;
-            dp[i] = 0.f;
-        }
+        for (int sb = 0; sb < NSUB; sb++) {
 #pragma unroll
-        for (int ks = 0; ks < C::KSTEPS; ks++) {
-            T8 a = as_vec<T8>(lds_read16(q_lds + SW::off(r, ks * 16 + 8 * g)));
-            s = mfma32(a, kreg[ks], s);
-        }
+            for (int q4 = 0; q4 < 4; q4++) {
+                const int ml0 = sb * 32 + 8 * q4 + 4 * g;  // first of 4 consecutive rows
+                const f32x4 lse4 = *reinterpret_cast<const f32x4*>(lse_lds + ml0);
+                const f32x4 del4 = *reinterpret_cast<const f32x4*>(delta_lds + ml0);
+                float bv[4] = {0.f, 0.f, 0.f, 0.f};
+                if constexpr (BIAS == 1) {
 #pragma unroll
-        for (int ks = 0; ks < C::KSTEPS; ks++) {
-            T8 a = as_vec<T8>(lds_read16(do_lds + SW::off(r, ks * 16 + 8 * g)));
-            dp = mfma32(a, vreg[ks], dp);
-        }
-
-        // ---- P and dS (flash_attention.py:281-306) ----
-        T8 pT[2], dsT[2];
+                    for (int e = 0; e < 4; e++) bv[e] = bt_lds[(ml0 + e) * 32 + r] ? 0.f : kMask;
+                } else if constexpr (BIAS == 2 || BIAS == 3) {
+                    typedef typename VecOf<E>::v4 B4;
+                    i16x4 raw = lds_read_tr4(reinterpret_cast<const E*>(bt_lds) + tr_offset(lane, ml0, 0, 32));
+                    B4 hv = __builtin_bit_cast(B4, raw);
 #pragma unroll
-        for (int q4 = 0; q4 < 4; q4++) {
-            const f32x4 lse4 = *reinterpret_cast<const f32x4*>(lse_lds + 8 * q4 + 4 * g);
-            const f32x4 del4 = *reinterpret_cast<const f32x4*>(delta_lds + 8 * q4 + 4 * g);
+                    for (int e = 0; e < 4; e++) bv[e] = (float)hv[e] * kLog2e;
+                } else if constexpr (BIAS == 4) {
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                const int i = q4 * 4 + e;
-                const int ml = 8 * q4 + 4 * g + e;  // row within the block
-                float x = __fmul_rn(s[i], qk_scale);
-                float add = (BIAS != 0) ? bv[i] : 0.f;
-                if (need_mask) {
-                    const int m = m0 + ml;
-                    float t = 0.f;
-                    if (m >= M || my_n >= N) t = kMask;
-                    if (CAUSAL && m < my_n) t += kMask;
-                    add = t + add;
+                    for (int e = 0; e < 4; e++) bv[e] = reinterpret_cast<const float*>(bt_lds)[(ml0 + e) * 32 + r] * kLog2e;
                 }
-                x = __fadd_rn(x, add);
-                const float pv = fast_exp2(x - lse4[e]);
-                const float dsv = pv * (dp[i] - del4[e]);
-                pT[i >> 3][i & 7] = (T)pv;
-                dsT[i >> 3][i & 7] = (T)dsv;
-                ds_lds[ml * DSS + wave * 32 + r] = (T)dsv;
-                if (DBIAS) {
-                    const int m = m0 + ml;
-                    if (m < M && my_n < N) dbp[(int64_t)m * p.sdbias.m + (int64_t)my_n * p.sdbias.n] = (E)dsv;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const int i = q4 * 4 + e;
+                    const int m = m0 + ml0 + e;
+                    float x = __fmul_rn(s[sb][i], qk_scale);
+                    float add = bv[e];
+                    if (need_mask) {
+                        const bool oob = (m >= M) || (my_n >= N);
+                        float t = oob ? kMask : 0.f;
+                        if (CAUSAL) t += (m < my_n) ? kMask : 0.f;
+                        if (BIAS != 0) add = oob ? kMask : add;
+                        add = t + add;
+                    }
+                    x = __fadd_rn(x, add);
+                    const float pv = fast_exp2(x - lse4[e]);
+                    const float dsv = pv * (dp[sb][i] - del4[e]);
+                    pT[sb][i >> 3][i & 7] = (T)pv;
+                    dsT[sb][i >> 3][i & 7] = (T)dsv;
+                    ds_lds[(ml0 + e) * DSS + wave * 32 + r] = (T)dsv;
+                    if constexpr (DBIAS && !DB_VIA_LDS) {
+                        if (m < M && my_n < N) dbp[(int64_t)m * p.sdbias.m + (int64_t)my_n * p.sdbias.n] = (E)dsv;
+                    }
                 }
             }
         }
 
         // ---- dV^T += dO^T P and dK^T += Q^T dS ----
 #pragma unroll
-        for (int kk = 0; kk < 2; kk++) {
+        for (int sb = 0; sb < NSUB; sb++) {
 #pragma unroll
-            for (int db = 0; db < C::DB; db++) {
-                T8 a = SW::template col8<T8>(do_lds, lane, kk * 16, db * 32);
-                dv_acc[db] = mfma32(a, pT[kk], dv_acc[db]);
-            }
+            for (int kk = 0; kk < 2; kk++) {
 #pragma unroll
-            for (int db = 0; db < C::DB; db++) {
-                T8 a = SW::template col8<T8>(q_lds, lane, kk * 16, db * 32);
-                dk_acc[db] = mfma32(a, dsT[kk], dk_acc[db]);
+                for (int db = 0; db < C::DB; db++) {
+                    T8 a = SW::template col8<T8>(do_lds, lane, sb * 32 + kk * 16, db * 32);
+                    dv_acc[db] = mfma32(a, pT[sb][kk], dv_acc[db]);
+                }
+#pragma unroll
+                for (int db = 0; db < C::DB; db++) {
+                    T8 a = SW::template col8<T8>(q_lds, lane, sb * 32 + kk * 16, db * 32);
+                    dk_acc[db] = mfma32(a, dsT[sb][kk], dk_acc[db]);
+                }
             }
         }
 
-        __syncthreads();  // the dS tile of all 128 keys is complete
+        // next block's tiles go into the other buffer while this one is still being read
+        if (mb + 1 < n_mblocks) stage(buf ^ 1);
+        __syncthreads();  // the dS tile of all 128 keys is complete; the next tiles are visible
 
-        // ---- dQ block (32 rows x 32 head-dim columns) += dS K ----
-        if (dq_active) {
-            f32x16 dq;
+        // ---- dBias rows of this wave's 32 keys, 16 bytes per lane, out of the dS tile ----
+        if constexpr (DB_VIA_LDS) {
 #pragma unroll
-            for (int i = 0; i < 16; i++) dq[i] = 0.f;
-#pragma unroll
-            for (int ks = 0; ks < BN / 16; ks++) {
-                T8 a = as_vec<T8>(lds_read16(ds_lds + r * DSS + ks * 16 + 8 * g));
-                dq = mfma32(a, ktreg[ks], dq);
+            for (int it = 0; it < (BMI * 4) / 64; it++) {
+                const int c = it * 64 + lane;
+                const int row = c >> 2, ch = c & 3;
+                const int m = m0 + row, nn = nw + ch * 8;
+                if (m < M && nn < N) {
+                    const T* src = ds_lds + row * DSS + wave * 32 + ch * 8;
+                    E* dst = dbp + (int64_t)m * p.sdbias.m + (int64_t)nn * p.sdbias.n;
+                    if (dbias_vec && nn + 8 <= N) {
+                        gst16(dst, lds_read16(src));
+                    } else {
+                        for (int e = 0; e < 8; e++)
+                            if (nn + e < N) dst[(int64_t)e * p.sdbias.n] = __builtin_bit_cast(E, src[e]);
+                    }
+                }
             }
-            const int d = dq_db * 32 + r;
-            if (d < D) {
+        }
+
+        // ---- dQ blocks (32 rows x 32 head-dim columns each) += dS K ----
+        if (dq_active) {
 #pragma unroll
-                for (int i = 0; i < 16; i++) {
-                    const int m = m0 + 8 * (i >> 2) + 4 * g + (i & 3);
-                    if (m < M)
-                        __hip_atomic_fetch_add(dqap + (int64_t)m * D + d, dq[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for (int j = 0; j < C::BPW; j++) {
+                const int sb = (dq_first + j) % NSUB;
+                f32x16 dq;
+#pragma unroll
+                for (int i = 0; i < 16; i++) dq[i] = 0.f;
+#pragma unroll
+                for (int ks = 0; ks < BN / 16; ks++) {
+                    T8 a = as_vec<T8>(lds_read16(ds_lds + (sb * 32 + r) * DSS + ks * 16 + 8 * g));
+                    dq = mfma32(a, ktreg[ks], dq);
+                }
+                const int d = dq_db * 32 + r;
+                if (d < D) {
+#pragma unroll
+                    for (int i = 0; i < 16; i++) {
+                        const int m = m0 + sb * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
+                        if (m < M)
+                            __hip_atomic_fetch_add(dqap + (int64_t)m * D + d, dq[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
                 }
             }
         }

@@ -47,6 +47,8 @@ struct BwdParams {
     int B, H, M, N;
     float sm_scale;
     int n_ntiles;
+    int bias_vec;   // bias rows may be read with aligned 16-byte loads
+    int dbias_vec;  // dbias rows may be written with aligned 16-byte stores
 };
 
 }  // namespace fa

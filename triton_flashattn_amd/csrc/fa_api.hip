@@ -34,6 +34,8 @@ bool qkv_layout_ok(const void* ptr, const int64_t s[4], int nb, int ns, int nh) 
     if (nb > 1 && s[0] % 8 != 0) return false;
     if (ns > 1 && s[1] % 8 != 0) return false;
     if (nh > 1 && s[2] % 8 != 0) return false;
+    // the kernels form 32-bit byte offsets inside a tile of up to 128 rows
+    if (ns > 1 && (s[1] < 0 || s[1] >= (1 << 23))) return false;
     return true;
 }
 
@@ -59,6 +61,8 @@ bool bias_vec_ok(const void* ptr, const int64_t s[4], const fa_problem& p) {
     if (p.B > 1 && (s[0] * es) % 16 != 0) return false;
     if (p.H > 1 && (s[1] * es) % 16 != 0) return false;
     if (p.M > 1 && (s[2] * es) % 16 != 0) return false;
+    // one (batch, head) slice is addressed through a 32-bit buffer descriptor
+    if (s[2] < 0 || ((int64_t)(p.M - 1) * s[2] + p.N) * es >= (1ll << 31)) return false;
     return true;
 }
 

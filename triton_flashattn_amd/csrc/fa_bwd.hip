@@ -28,33 +28,6 @@
 
 namespace fa {
 
-// Row-major LDS tile of 16-bit elements, D per row, no padding; 16-byte chunks are XOR-swizzled
-// by a function of the row so that both 16-byte row reads (lane = row) and 4-row column gathers
-// (ds_read_b64_tr_b16) are free of bank conflicts.
-template <int D> struct Swz {
-    static constexpr int CPR = D / 8;
-    __device__ static __forceinline__ int f(int row) {
-        if (CPR >= 16) return ((row & 3) << 2) | ((row >> 2) & 3);
-        if (CPR == 8) return (((row >> 1) & 1) << 2) | ((row >> 2) & 3);
-        if (CPR == 4) return (row >> 2) & 3;
-        return (row >> 3) & 1;
-    }
-    __device__ static __forceinline__ int off(int row, int col) {
-        return row * D + ((((col >> 3) ^ f(row)) << 3) | (col & 7));
-    }
-    // 8 k-slots gathered down column col0 + lane%32: rows row0 + 4g + {0..3}, row0 + 8 + 4g + {0..3}
-    template <typename V8, typename T>
-    __device__ static __forceinline__ V8 col8(const T* tile, int lane, int row0, int col0) {
-        const int g = lane >> 5, s = lane & 15;
-        const int row = row0 + 4 * g + (s >> 2);
-        const int col = (col0 + ((lane >> 4) & 1) * 16 + (s & 3) * 4) & (D - 1);
-        i16x4 lo = lds_read_tr4(tile + off(row, col));
-        i16x4 hi = lds_read_tr4(tile + off(row + 8, col));
-        typedef short i16x8 __attribute__((ext_vector_type(8)));
-        return __builtin_bit_cast(V8, (i16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-    }
-};
-
 // ---------------------------------------------------------------------------------------------
 template <typename T, int D>
 __global__ __launch_bounds__(256) void fa_bwd_prep_kernel(const BwdParams p) {

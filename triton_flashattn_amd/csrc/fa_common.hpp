@@ -92,7 +92,55 @@ __device__ __forceinline__ V8 lds_read_col8(const T* tile, int lane, int row0, i
     return __builtin_bit_cast(V8, v);
 }
 
+// Row-major LDS tile of 16-bit elements, D per row, no padding; the 16-byte chunks of a row are
+// XOR-swizzled by a function of the row so that both 16-byte row reads (lane = row) and 4-row
+// column gathers (ds_read_b64_tr_b16) are free of bank conflicts.
+template <int D> struct Swz {
+    static constexpr int CPR = D / 8;  // chunks per row
+    __device__ static __forceinline__ int f(int row) {
+        if (CPR >= 16) return ((row & 3) << 2) | ((row >> 2) & 3);
+        if (CPR == 8) return (((row >> 1) & 1) << 2) | ((row >> 2) & 3);
+        if (CPR == 4) return (row >> 2) & 3;
+        return (row >> 3) & 1;
+    }
+    __device__ static __forceinline__ int off(int row, int col) {
+        return row * D + ((((col >> 3) ^ f(row)) << 3) | (col & 7));
+    }
+    // 8 k-slots gathered down column col0 + lane%32: rows row0 + 4g + {0..3}, row0 + 8 + 4g + {0..3}
+    template <typename V8, typename T>
+    __device__ static __forceinline__ V8 col8(const T* tile, int lane, int row0, int col0) {
+        const int g = lane >> 5, s = lane & 15;
+        const int row = row0 + 4 * g + (s >> 2);
+        const int col = (col0 + ((lane >> 4) & 1) * 16 + (s & 3) * 4) & (D - 1);
+        i16x4 lo = lds_read_tr4(tile + off(row, col));
+        i16x4 hi = lds_read_tr4(tile + off(row + 8, col));
+        typedef short i16x8 __attribute__((ext_vector_type(8)));
+        return __builtin_bit_cast(V8, (i16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    }
+};
+
 // ---- global access ------------------------------------------------------------------------
+// global_load_lds_dwordx4: lane l copies the 16 bytes at `src` (per lane) to lds_base + 16 l
+// (lds_base is wave-uniform) without passing through registers; completion counts on vmcnt.
+__device__ __forceinline__ void g2lds16(const void* src, void* lds_base) {
+    __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)src,
+                                     (void __attribute__((address_space(3)))*)lds_base, 16, 0, 0);
+}
+
+// Raw buffer view of `bytes` bytes at `base` (16-byte aligned): loads beyond the end return 0 and
+// stores beyond the end are dropped.  The range check works on whole dwords, so the length is
+// rounded up to the dword that holds the last byte (still inside the aligned allocation); a
+// caller that stores through the view must not address the rounding slack.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_buffer(const void* base, int64_t bytes) {
+    const int64_t cap = 0xfffffffcll;
+    bytes = (bytes + 3) & ~(int64_t)3;
+    const unsigned n = bytes < 0 ? 0u : (unsigned)(bytes > cap ? cap : bytes);
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)n, 0x00020000);
+}
+__device__ __forceinline__ i32x4 buf_load16(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
+    return __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
+}
+
 __device__ __forceinline__ i32x4 gld16(const void* p) { return *reinterpret_cast<const i32x4*>(p); }
 __device__ __forceinline__ void gst16(void* p, i32x4 v) { *reinterpret_cast<i32x4*>(p) = v; }
 

@@ -14,6 +14,8 @@
 // ds_read_b64_tr_b16.  The bias tile of a wave (32 rows x 64 keys) is staged through a
 // wave-private LDS region with 16-byte coalesced global loads and read back in accumulator
 // layout (4 consecutive keys per read).
+#include <type_traits>
+
 #include "fa_common.hpp"
 #include "fa_params.hpp"
 
@@ -22,20 +24,22 @@ namespace fa {
 template <int D, int BIAS> struct FwdCfg {
     static constexpr int BM = 128, BN = 64, NT = 256;
     static constexpr int DP = D < 32 ? 32 : D;       // head dim padded to one 32-wide MFMA block
-    static constexpr int KS = D + 8;                 // K tile row stride (elements): 16 B skew
-    static constexpr int VS = DP + 32;               // V tile row stride: 64 B skew (transposed reads)
-    static constexpr int OS = DP + 8;                // O staging row stride
+    static constexpr int OS = DP + 8;                // O staging row stride (elements)
     static constexpr int CPR = D / 8;                // 16-byte chunks per row
-    static constexpr int NCH = (BN * CPR + NT - 1) / NT;  // chunks per thread per K (or V) tile
+    static constexpr int TILE_CHUNKS = BN * CPR;     // 16-byte chunks per K (or V) tile
+    static constexpr int NCH = (TILE_CHUNKS + NT - 1) / NT;  // direct-to-LDS copies per thread per tile
     static constexpr int KSTEPS = D / 16;            // MFMA k-steps of Q K^T
     static constexpr int DB = DP / 32;               // 32-wide blocks of the head dim
     static constexpr int ES = BIAS == 0 ? 0 : (BIAS == 1 ? 1 : (BIAS == 4 ? 4 : 2));
-    static constexpr int BROW = BIAS == 0 ? 0 : (ES == 1 ? 72 : (ES == 2 ? 136 : 272));  // bytes
+    static constexpr int BROW = 64 * ES;             // bias tile row: 64 keys, unpadded, chunk-swizzled
+    // 16-byte chunk c of bias row `row` is stored at chunk c ^ bswz(row)
+    __device__ static __forceinline__ int bswz(int row) {
+        return ES == 4 ? (row & 15) : (ES == 2 ? (row & 7) : ((row >> 2) & 3));
+    }
     static constexpr int BCH = 2 * ES;               // 16-byte bias chunks per lane per tile
-    static constexpr int K_BYTES = BN * KS * 2;
-    static constexpr int V_BYTES = BN * VS * 2;
+    static constexpr int TILE_BYTES = BN * D * 2;    // unpadded, swizzled
     static constexpr int O_BYTES = BM * OS * 2;
-    static constexpr int KV_BYTES = (K_BYTES + V_BYTES) > O_BYTES ? (K_BYTES + V_BYTES) : O_BYTES;
+    static constexpr int KV_BYTES = 4 * TILE_BYTES > O_BYTES ? 4 * TILE_BYTES : O_BYTES;  // K[2], V[2]
     static constexpr int BIAS_BYTES = 4 * 32 * BROW;
     static constexpr int LDS_BYTES = KV_BYTES + BIAS_BYTES;
     // two work-groups per CU whenever registers allow it
@@ -45,14 +49,13 @@ template <int D, int BIAS> struct FwdCfg {
 template <typename T, int D, int BIAS, bool CAUSAL>
 __global__ __launch_bounds__(256, (FwdCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_kernel(const FwdParams p) {
     typedef FwdCfg<D, BIAS> C;
+    typedef Swz<D> SW;
     typedef typename VecOf<T>::v8 T8;
     typedef typename VecOf<T>::v4 T4;
     typedef typename BiasElem<BIAS>::type E;
-    constexpr int BM = C::BM, BN = C::BN, KS = C::KS, VS = C::VS, OS = C::OS, CPR = C::CPR;
+    constexpr int BM = C::BM, BN = C::BN, OS = C::OS, CPR = C::CPR;
 
     __shared__ __align__(16) unsigned char smem[C::LDS_BYTES];
-    T* k_lds = reinterpret_cast<T*>(smem);
-    T* v_lds = reinterpret_cast<T*>(smem + C::K_BYTES);
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
@@ -68,18 +71,13 @@ __global__ __launch_bounds__(256, (FwdCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_ker
     const int my_m = mw + r;
 
     const T* qp = reinterpret_cast<const T*>(p.q) + (int64_t)b * p.sq.b + (int64_t)h * p.sq.h;
-    const T* kp = reinterpret_cast<const T*>(p.k) + (int64_t)b * p.sk.b + (int64_t)h * p.sk.h;
-    const T* vp = reinterpret_cast<const T*>(p.v) + (int64_t)b * p.sv.b + (int64_t)h * p.sv.h;
+    const char* kbase = reinterpret_cast<const char*>(reinterpret_cast<const T*>(p.k) + (int64_t)b * p.sk.b + (int64_t)h * p.sk.h);
+    const char* vbase = reinterpret_cast<const char*>(reinterpret_cast<const T*>(p.v) + (int64_t)b * p.sv.b + (int64_t)h * p.sv.h);
     const E* bp = nullptr;
     unsigned char* bias_lds = nullptr;
     if (BIAS != 0) {
         bp = reinterpret_cast<const E*>(p.bias) + (int64_t)b * p.sbias.b + (int64_t)h * p.sbias.h;
         bias_lds = smem + C::KV_BYTES + wave * 32 * C::BROW;
-    }
-
-    // V columns D..DP-1 (only when D < 32) are never loaded: keep them zero
-    if (D < C::DP) {
-        for (int i = tid; i < BN * VS; i += C::NT) v_lds[i] = (T)0.f;
     }
 
     // Q^T as B operand: column my_m, k = d
@@ -105,165 +103,223 @@ __global__ __launch_bounds__(256, (FwdCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_ker
 #pragma unroll
         for (int i = 0; i < 16; i++) o_acc[db][i] = 0.f;
 
-    i32x4 kreg[C::NCH], vreg[C::NCH];
-    i32x4 breg[C::BCH > 0 ? C::BCH : 1];
-
-    auto prefetch = [&](int j) {
+    // ---- K / V tiles: global -> LDS without passing through registers.  Chunk c of a tile
+    // (row c / CPR, LDS chunk c % CPR) is copied by thread c % 256 in copy c / 256; the LDS chunk
+    // holds global chunk (c % CPR) ^ f(row), which is the swizzle the readers expect.
+    unsigned koff[C::NCH], voff[C::NCH];  // byte offsets of this lane's source chunks in a full tile
+#pragma unroll
+    for (int it = 0; it < C::NCH; it++) {
+        const int c = it * C::NT + tid;
+        const int row = c / CPR, src = (c % CPR) ^ SW::f(row);
+        koff[it] = (unsigned)(row * (int)p.sk.s * 2 + src * 16);
+        voff[it] = (unsigned)(row * (int)p.sv.s * 2 + src * 16);
+    }
+    auto issue_tile = [&](int j, int buf) {
         const int n0 = j * BN;
+        const char* kt = kbase + (int64_t)n0 * p.sk.s * 2;
+        const char* vt = vbase + (int64_t)n0 * p.sv.s * 2;
+        unsigned char* k_dst = smem + buf * C::TILE_BYTES;
+        unsigned char* v_dst = smem + (2 + buf) * C::TILE_BYTES;
+        const bool full = n0 + BN <= N;
 #pragma unroll
         for (int it = 0; it < C::NCH; it++) {
-            int c = it * C::NT + tid;
-            int row = c / CPR, ch = c % CPR;
-            bool ok = (c < BN * CPR) && (n0 + row < N);
-            i32x4 z = {0, 0, 0, 0};
-            kreg[it] = ok ? gld16(kp + (int64_t)(n0 + row) * p.sk.s + ch * 8) : z;
-            vreg[it] = ok ? gld16(vp + (int64_t)(n0 + row) * p.sv.s + ch * 8) : z;
-        }
-        if (BIAS != 0) {
-            if (p.bias_vec && n0 + BN <= N) {
-                constexpr int CH_ROW = 4 * C::ES;  // 16-byte chunks per 64-key row
-#pragma unroll
-                for (int it = 0; it < C::BCH; it++) {
-                    int c = it * 64 + lane;
-                    int row = c / CH_ROW, ch = c % CH_ROW;
-                    i32x4 z = {0, 0, 0, 0};
-                    const unsigned char* src = reinterpret_cast<const unsigned char*>(
-                        bp + (int64_t)(mw + row) * p.sbias.m + n0) + ch * 16;
-                    breg[it] = (mw + row < M) ? gld16(src) : z;
+            const int c0 = it * C::NT + wave * 64;  // first chunk of this wave's copy
+            if (c0 < C::TILE_CHUNKS) {
+                unsigned ko = koff[it], vo = voff[it];
+                if (!full) {  // rows past the last key re-read the last key; the scores are masked
+                    const int c = c0 + lane;
+                    int row = c / CPR;
+                    const int src = (c % CPR) ^ SW::f(row);
+                    row = row < N - n0 ? row : N - n0 - 1;
+                    ko = (unsigned)(row * (int)p.sk.s * 2 + src * 16);
+                    vo = (unsigned)(row * (int)p.sv.s * 2 + src * 16);
                 }
+                g2lds16(kt + ko, k_dst + c0 * 16);
+                g2lds16(vt + vo, v_dst + c0 * 16);
             }
         }
     };
 
-    if (n_tiles > 0) prefetch(0);
-
-    for (int j = 0; j < n_tiles; j++) {
-        const int n0 = j * BN;
-        __syncthreads();  // every wave is done reading the previous tile
+    // ---- bias tile of this wave (32 rows x 64 keys): global -> registers one tile ahead ----
+    i32x4 breg[C::BCH > 0 ? C::BCH : 1];
+    int boff[C::BCH > 0 ? C::BCH : 1];
+    __amdgpu_buffer_rsrc_t brsrc = make_buffer(nullptr, 0);
+    if constexpr (BIAS != 0) {
+        constexpr int CH_ROW = 4 * C::ES;  // 16-byte chunks per 64-key row
 #pragma unroll
-        for (int it = 0; it < C::NCH; it++) {
-            int c = it * C::NT + tid;
-            int row = c / CPR, ch = c % CPR;
-            if (c < BN * CPR) {
-                lds_write16(k_lds + row * KS + ch * 8, kreg[it]);
-                lds_write16(v_lds + row * VS + ch * 8, vreg[it]);
+        for (int it = 0; it < C::BCH; it++) {
+            const int c = it * 64 + lane;
+            boff[it] = (c / CH_ROW) * (int)p.sbias.m * C::ES + (c % CH_ROW) * 16;
+        }
+        // everything from the first row of this wave to the end of the (b, h) slice
+        brsrc = make_buffer(bp + (int64_t)mw * p.sbias.m, ((int64_t)(M - 1 - mw) * p.sbias.m + N) * C::ES);
+    }
+    auto prefetch_bias = [&](int j) {
+        if constexpr (BIAS != 0) {
+            if (p.bias_vec) {
+#pragma unroll
+                for (int it = 0; it < C::BCH; it++) breg[it] = buf_load16(brsrc, boff[it], j * BN * C::ES);
             }
         }
-        if (BIAS != 0) {
-            if (p.bias_vec && n0 + BN <= N) {
-                constexpr int CH_ROW = 4 * C::ES;
+    };
+
+    if (n_tiles > 0) {
+        issue_tile(0, 0);
+        prefetch_bias(0);
+    }
+
+#pragma unroll 1
+    for (int j = 0; j < n_tiles; j++) {
+        const int n0 = j * BN;
+        const int buf = j & 1;
+        const T* k_lds = reinterpret_cast<const T*>(smem + buf * C::TILE_BYTES);
+        const T* v_lds = reinterpret_cast<const T*>(smem + (2 + buf) * C::TILE_BYTES);
+        __builtin_amdgcn_s_waitcnt(0);  // this thread's copies of tile j (and its bias chunks) have landed
+        if constexpr (BIAS != 0) {
+            if (p.bias_vec) {
 #pragma unroll
                 for (int it = 0; it < C::BCH; it++) {
-                    int c = it * 64 + lane;
-                    int row = c / CH_ROW, ch = c % CH_ROW;
-                    i32x2* dst = reinterpret_cast<i32x2*>(bias_lds + row * C::BROW + ch * 16);
-                    i32x2 lo = {breg[it][0], breg[it][1]}, hi = {breg[it][2], breg[it][3]};
-                    dst[0] = lo;
-                    dst[1] = hi;
+                    constexpr int CH_ROW = 4 * C::ES;
+                    const int c = it * 64 + lane;
+                    const int row = c / CH_ROW;
+                    lds_write16(bias_lds + row * C::BROW + (((c % CH_ROW) ^ C::bswz(row)) << 4), breg[it]);
                 }
             } else {
-                // ragged or unaligned bias: one element per lane per row, any strides
+                // unaligned bias rows or non-unit key stride: one element per lane per row
 #pragma unroll 1
                 for (int row = 0; row < 32; row++) {
                     int n = n0 + lane;
                     E val = (E)0.f;
                     if (mw + row < M && n < N)
                         val = bp[(int64_t)(mw + row) * p.sbias.m + (int64_t)n * p.sbias.n];
-                    *reinterpret_cast<E*>(bias_lds + row * C::BROW + lane * C::ES) = val;
+                    const int byte = lane * C::ES;
+                    *reinterpret_cast<E*>(bias_lds + row * C::BROW + (((byte >> 4) ^ C::bswz(row)) << 4) + (byte & 15)) = val;
                 }
             }
         }
-        __syncthreads();
-        if (j + 1 < n_tiles) prefetch(j + 1);
+        __syncthreads();  // tile j is complete in LDS; nobody still reads the buffer of tile j - 1
+        if (j + 1 < n_tiles) {
+            issue_tile(j + 1, buf ^ 1);
+            prefetch_bias(j + 1);
+        }
 
-        // tiles entirely above this wave's diagonal contribute nothing
-        if (CAUSAL && n0 > mw + 31) continue;
-        const bool need_mask = (n0 + BN > N) || (CAUSAL && n0 + BN - 1 > mw);
-
-        // ---- S^T = K Q^T : s[nb][i] is key n0 + 32 nb + 8 (i/4) + 4 g + i%4, query my_m ----
-        f32x16 s[2];
+        // The 64-key tile is consumed as two 32-key halves, each with its own softmax step, so
+        // that only one 32 x 32 score block is live at a time.
 #pragma unroll
         for (int nb = 0; nb < 2; nb++) {
+            const int nh = nb * 32;  // first key of this half inside the tile
+            __builtin_amdgcn_sched_barrier(0);  // keep the halves apart: one score block live at a time
+            // halves entirely above this wave's diagonal contribute nothing
+            if (CAUSAL && n0 + nh > mw + 31) continue;
+            if (n0 + nh >= N) continue;
+            const bool need_mask = (n0 + nh + 32 > N) || (CAUSAL && n0 + nh + 31 > mw);
+
+            // ---- S^T = K Q^T : s[i] is key n0 + nh + 8 (i/4) + 4 g + i%4, query my_m ----
+            f32x16 s;
 #pragma unroll
-            for (int i = 0; i < 16; i++) s[nb][i] = 0.f;
+            for (int i = 0; i < 16; i++) s[i] = 0.f;
 #pragma unroll
             for (int ks = 0; ks < C::KSTEPS; ks++) {
-                T8 a = as_vec<T8>(lds_read16(k_lds + (nb * 32 + r) * KS + ks * 16 + 8 * g));
-                s[nb] = mfma32(a, qreg[ks], s[nb]);
+                T8 a = as_vec<T8>(lds_read16(k_lds + SW::off(nh + r, ks * 16 + 8 * g)));
+                s = mfma32(a, qreg[ks], s);
             }
-        }
 
-        // ---- scale, bias, masks (additive -1e6 in log2 units, flash_attention.py:39-53) ----
-        float mx = -INFINITY;
-#pragma unroll
-        for (int nb = 0; nb < 2; nb++) {
-#pragma unroll
-            for (int q4 = 0; q4 < 4; q4++) {
-                const int nl = nb * 32 + 8 * q4 + 4 * g;  // first of 4 consecutive keys
-                float bv[4] = {0.f, 0.f, 0.f, 0.f};
-                if constexpr (BIAS == 1) {
-                    unsigned int w = *reinterpret_cast<const unsigned int*>(bias_lds + r * C::BROW + nl);
-#pragma unroll
-                    for (int e = 0; e < 4; e++) bv[e] = ((w >> (8 * e)) & 0xffu) ? 0.f : kMask;
-                } else if constexpr (BIAS == 2 || BIAS == 3) {
-                    typedef typename VecOf<E>::v4 B4;
-                    B4 hv = *reinterpret_cast<const B4*>(bias_lds + r * C::BROW + nl * 2);
-#pragma unroll
-                    for (int e = 0; e < 4; e++) bv[e] = (float)hv[e] * kLog2e;
-                } else if constexpr (BIAS == 4) {
-                    f32x4 w = *reinterpret_cast<const f32x4*>(bias_lds + r * C::BROW + nl * 4);
-#pragma unroll
-                    for (int e = 0; e < 4; e++) bv[e] = w[e] * kLog2e;
-                }
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const int i = q4 * 4 + e;
-                    float x = __fmul_rn(s[nb][i], qk_scale);
-                    float add = bv[e];
-                    if (need_mask) {
-                        const int n = n0 + nl + e;
-                        float t = 0.f;
-                        if (n >= N) t = kMask;
-                        if (CAUSAL && my_m < n) t += kMask;
-                        if (BIAS != 0 && n >= N) add = kMask;  // out-of-range bias reads as masked
-                        add = t + add;
+            // ---- online softmax step.  `masked` tiles (ragged edge, causal diagonal) and a
+            // non-positive scale follow the reference's arithmetic term by term: scaled score,
+            // plus additive -1e6 terms in log2 units, plus bias (flash_attention.py:39-53).  Interior
+            // tiles skip the mask terms and fold the scale into the exponent.
+            // The running maximum m_i is only raised when a tile exceeds it by more than 2^8: the
+            // reference point of the exponentials is arbitrary (out = acc / l and LSE = m + log2 l
+            // do not depend on it), so a stale one costs nothing but saves rescaling O every tile.
+            T8 pb[2];
+            auto softmax_step = [&](auto masked_tag) {
+                constexpr bool MASKED = decltype(masked_tag)::value;
+                float mx = -INFINITY;
+                {
+    #pragma unroll
+                    for (int q4 = 0; q4 < 4; q4++) {
+                        const int nl = nh + 8 * q4 + 4 * g;  // first of 4 consecutive keys
+                        float bv[4] = {0.f, 0.f, 0.f, 0.f};       // bias in natural units
+                        bool keep[4] = {true, true, true, true};
+                        if constexpr (BIAS == 1) {
+                            unsigned int w = *reinterpret_cast<const unsigned int*>(bias_lds + r * C::BROW + (((nl >> 4) ^ C::bswz(r)) << 4) + (nl & 15));
+    #pragma unroll
+                            for (int e = 0; e < 4; e++) keep[e] = ((w >> (8 * e)) & 0xffu) != 0;
+                        } else if constexpr (BIAS == 2 || BIAS == 3) {
+                            typedef typename VecOf<E>::v4 B4;
+                            B4 hv = *reinterpret_cast<const B4*>(bias_lds + r * C::BROW + (((nl >> 3) ^ C::bswz(r)) << 4) + ((nl * 2) & 15));
+    #pragma unroll
+                            for (int e = 0; e < 4; e++) bv[e] = (float)hv[e];
+                        } else if constexpr (BIAS == 4) {
+                            f32x4 w = *reinterpret_cast<const f32x4*>(bias_lds + r * C::BROW + (((nl >> 2) ^ C::bswz(r)) << 4));
+    #pragma unroll
+                            for (int e = 0; e < 4; e++) bv[e] = w[e];
+                        }
+    #pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            const int i = q4 * 4 + e;
+                            float x;
+                            if constexpr (MASKED) {
+                                x = __fmul_rn(s[i], qk_scale);
+                                const int n = n0 + nl + e;
+                                float t = (n >= N) ? kMask : 0.f;
+                                if (CAUSAL) t += (my_m < n) ? kMask : 0.f;
+                                float add = 0.f;
+                                if (BIAS == 1) add = keep[e] ? 0.f : kMask;
+                                if (BIAS >= 2) add = __fmul_rn(bv[e], kLog2e);
+                                if (BIAS != 0) add = (n >= N) ? kMask : add;  // out-of-range bias reads as masked
+                                x = __fadd_rn(x, __fadd_rn(t, add));
+                            } else if constexpr (BIAS == 0) {
+                                x = s[i];                                    // raw score, scale folded below
+                            } else if constexpr (BIAS == 1) {
+                                x = keep[e] ? s[i] * qk_scale : s[i] * qk_scale + kMask;
+                            } else {
+                                x = s[i] * p.sm_scale + bv[e];               // natural units
+                            }
+                            s[i] = x;
+                            mx = fmaxf(mx, x);
+                        }
                     }
-                    x = __fadd_rn(x, add);
-                    s[nb][i] = x;
-                    mx = fmaxf(mx, x);
                 }
-            }
-        }
-        mx = pair_max(mx);
-        const float m_new = fmaxf(m_i, mx);
-        const float alpha = fast_exp2(m_i - m_new);
-        m_i = m_new;
-        float rs = 0.f;
-        T8 pb[2][2];
-#pragma unroll
-        for (int nb = 0; nb < 2; nb++) {
-#pragma unroll
-            for (int i = 0; i < 16; i++) {
-                float pv = fast_exp2(s[nb][i] - m_new);
-                rs += pv;
-                pb[nb][i >> 3][i & 7] = (T)pv;
-            }
-        }
-        l_i = l_i * alpha + rs;  // per-lane partial sum; the two halves are added at the end
-#pragma unroll
-        for (int db = 0; db < C::DB; db++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) o_acc[db][i] *= alpha;
+                // units of x: log2 (MASKED, bool bias), raw dot product (no bias), natural (float bias)
+                constexpr bool RAW = !MASKED && BIAS == 0;
+                constexpr bool NAT = !MASKED && BIAS >= 2;
+                const float to_log2 = RAW ? qk_scale : (NAT ? kLog2e : 1.f);
+                mx = pair_max(mx) * to_log2;
+                const bool raise = mx > m_i + 8.f;
+                if (__builtin_amdgcn_ballot_w64(raise) != 0) {
+                    const float m_new = raise ? mx : m_i;
+                    const float alpha = fast_exp2(m_i - m_new);
+                    m_i = m_new;
+                    l_i *= alpha;
+    #pragma unroll
+                    for (int db = 0; db < C::DB; db++)
+    #pragma unroll
+                        for (int i = 0; i < 16; i++) o_acc[db][i] *= alpha;
+                }
+                float rs = 0.f;
+                {
+    #pragma unroll
+                    for (int i = 0; i < 16; i++) {
+                        float pv;
+                        if constexpr (RAW || NAT) pv = fast_exp2(__builtin_fmaf(s[i], to_log2, -m_i));
+                        else pv = fast_exp2(s[i] - m_i);
+                        rs += pv;
+                        pb[i >> 3][i & 7] = (T)pv;
+                    }
+                }
+                l_i += rs;  // per-lane partial sum; the two halves are added at the end
+            };
+            if (need_mask || !(qk_scale > 0.f)) softmax_step(std::true_type{});
+            else softmax_step(std::false_type{});
 
-        // ---- O^T += V^T P^T : A = V^T gathered down the columns of the V tile ----
-#pragma unroll
-        for (int nb = 0; nb < 2; nb++) {
+            // ---- O^T += V^T P^T : A = V^T gathered down the columns of the V tile ----
 #pragma unroll
             for (int kk = 0; kk < 2; kk++) {
 #pragma unroll
                 for (int db = 0; db < C::DB; db++) {
-                    T8 a = lds_read_col8<T8>(v_lds, lane, nb * 32 + kk * 16, db * 32, VS);
-                    o_acc[db] = mfma32(a, pb[nb][kk], o_acc[db]);
+                    T8 a = SW::template col8<T8>(v_lds, lane, nh + kk * 16, db * 32);
+                    o_acc[db] = mfma32(a, pb[kk], o_acc[db]);
                 }
             }
         }

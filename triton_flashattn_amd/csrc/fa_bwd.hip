@@ -84,34 +84,48 @@ __global__ __launch_bounds__(256) void fa_bwd_dq_kernel(const BwdParams p) {
 
 // ---------------------------------------------------------------------------------------------
 template <int D, int BIAS> struct BwdCfg {
-    static constexpr int BN = 128, BMI = 64, NSUB = BMI / 32, NT = 256;
+    static constexpr int BN = 128, NT = 512;
+    static constexpr int NSUB = D <= 64 ? 2 : 1;     // 32-row sub-blocks of a query block
+    static constexpr int BMI = 32 * NSUB;
     static constexpr int DP = D < 32 ? 32 : D;
     static constexpr int DB = DP / 32;
     static constexpr int KSTEPS = D / 16;
     static constexpr int CPR = D / 8;
-    static constexpr int NCH = (BMI * CPR + NT - 1) / NT;  // 16-byte chunks per thread per Q (or dO) block
+    static constexpr int QCH = (BMI * CPR + NT - 1) / NT;  // 16-byte chunks per thread per Q (or dO) block
     static constexpr int DSS = BN + 8;                     // dS tile row stride (elements)
     static constexpr int KTS = DP + 32;                    // one-time K tile (column gathers) row stride
     static constexpr int ES = BIAS == 0 ? 0 : (BIAS == 1 ? 1 : (BIAS == 4 ? 4 : 2));
-    static constexpr int BCH = (BMI * 32 * ES) / (64 * 16);  // 16-byte bias chunks per lane per block
+    static constexpr int EPC = ES > 0 ? 16 / ES : 8;       // bias elements per 16-byte chunk
     static constexpr int BCPR = 2 * ES;                    // 16-byte chunks per 32-key bias row
+    static constexpr int BCH = (BMI * BCPR + 63) / 64;     // bias chunks per lane per block
     static constexpr int Q_BYTES = BMI * D * 2;
     static constexpr int DS_BYTES = BMI * DSS * 2;
+    static constexpr int P_BYTES = 4 * NSUB * 64 * 64;     // P hand-off: 16 floats per lane per sub-block
     static constexpr int STAT_BYTES = 2 * BMI * 4;
     static constexpr int BT_BYTES = BMI * 32 * ES;         // wave-private bias tile
     static constexpr int OFF_DO = 2 * Q_BYTES;
     static constexpr int OFF_DS = 4 * Q_BYTES;
-    static constexpr int OFF_STAT = OFF_DS + 2 * DS_BYTES;
+    static constexpr int OFF_P = OFF_DS + 2 * DS_BYTES;
+    static constexpr int OFF_STAT = OFF_P + P_BYTES;
     static constexpr int OFF_BIAS = OFF_STAT + 2 * STAT_BYTES;
     static constexpr int LOOP_BYTES = OFF_BIAS + 4 * BT_BYTES;
     static constexpr int KT_BYTES = BN * KTS * 2;
     static constexpr int LDS_BYTES = LOOP_BYTES > KT_BYTES ? LOOP_BYTES : KT_BYTES;
     static constexpr int NDQ = NSUB * DB;                  // 32 x 32 blocks of dQ per query block
-    static constexpr int BPW = NDQ >= 4 ? NDQ / 4 : 1;     // dQ blocks per wave
+    static constexpr int BPW = NDQ >= 4 ? NDQ / 4 : 1;     // dQ blocks per S-wave
 };
 
+// Work split inside a work-group of 8 waves.  Waves 0-3 ("S-waves") and waves 4-7 ("dP-waves")
+// pair up on the four 32-key blocks of the tile (waves w and w + 4 run on the same SIMD):
+//   S-wave : S = Q K^T, P = 2^(S*scale + bias - LSE)  -> hands P to its partner through LDS,
+//            dV^T += dO^T P, and one 32-wide head-dim slice of dQ += dS K (all 128 keys)
+//   dP-wave: dP = dO V^T, dS = P (dP - delta) -> dS tile in LDS (+ dBias), dK^T += Q^T dS
+// A step handles one query block t and is cut in two by barriers so that in each half one wave
+// of a SIMD issues matrix instructions while the other does the exponentials / products:
+//   first half : S-wave: S(t), P(t)            dP-wave: dP(t), dK(t-1)
+//   second half: S-wave: dV(t), dQ(t-1)        dP-wave: dS(t), dBias(t)
 template <typename T, int D, int BIAS, bool CAUSAL, bool DBIAS>
-__global__ __launch_bounds__(256, 1) void fa_bwd_kernel(const BwdParams p) {
+__global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
     typedef BwdCfg<D, BIAS> C;
     typedef Swz<D> SW;
     typedef typename VecOf<T>::v8 T8;
@@ -119,21 +133,22 @@ __global__ __launch_bounds__(256, 1) void fa_bwd_kernel(const BwdParams p) {
     typedef typename BiasElem<BIAS>::type E;
     constexpr int BN = C::BN, BMI = C::BMI, CPR = C::CPR, DSS = C::DSS, NSUB = C::NSUB;
     // dBias leaves through the dS tile (16-byte row stores) when it has the element type of dS
-    constexpr bool DB_VIA_LDS = DBIAS && ((BIAS == 2 && sizeof(T) == 2 && __is_same(T, _Float16)) ||
-                                          (BIAS == 3 && __is_same(T, __bf16)));
+    constexpr bool DB_VIA_LDS = DBIAS && ((BIAS == 2 && __is_same(T, _Float16)) || (BIAS == 3 && __is_same(T, __bf16)));
 
     __shared__ __align__(16) unsigned char smem[C::LDS_BYTES];
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
     const int r = lane & 31, g = lane >> 5;
+    const bool s_wave = wave < 4;  // role
+    const int kb = wave & 3;       // 32-key block of this wave
 
     int nt, bh;
     decode_block(blockIdx.x, p.n_ntiles, p.B * p.H, nt, bh);
     const int b = bh / p.H, h = bh % p.H;
     const int M = p.M, N = p.N;
     const int n0 = nt * BN;
-    const int nw = n0 + wave * 32;
+    const int nw = n0 + kb * 32;
     const int my_n = nw + r;
 
     const T* qp = reinterpret_cast<const T*>(p.q) + (int64_t)b * p.sq.b + (int64_t)h * p.sq.h;
@@ -147,29 +162,29 @@ __global__ __launch_bounds__(256, 1) void fa_bwd_kernel(const BwdParams p) {
     E* dbp = nullptr;
     if (BIAS != 0) bp = reinterpret_cast<const E*>(p.bias) + (int64_t)b * p.sbias.b + (int64_t)h * p.sbias.h;
     if (DBIAS) dbp = reinterpret_cast<E*>(p.dbias) + (int64_t)b * p.sdbias.b + (int64_t)h * p.sdbias.h;
-    unsigned char* bt_lds = smem + C::OFF_BIAS + wave * C::BT_BYTES;
+    unsigned char* bt_lds = smem + C::OFF_BIAS + kb * C::BT_BYTES;
+    float* p_lds = reinterpret_cast<float*>(smem + C::OFF_P) + kb * NSUB * 64 * 16;
 
-    // ---- K and V of this wave's 32 keys as B operands (column my_n, k = d) ----
-    T8 kreg[C::KSTEPS], vreg[C::KSTEPS];
+    // ---- this wave's 32 keys as B operand (column my_n, k = d): K for an S-wave, V for a dP-wave
+    T8 opreg[C::KSTEPS];
+    {
+        const T* src = s_wave ? kp + (int64_t)my_n * p.sk.s : vp + (int64_t)my_n * p.sv.s;
 #pragma unroll
-    for (int ks = 0; ks < C::KSTEPS; ks++) {
-        i32x4 kr = {0, 0, 0, 0}, vr = {0, 0, 0, 0};
-        if (my_n < N) {
-            kr = gld16(kp + (int64_t)my_n * p.sk.s + ks * 16 + 8 * g);
-            vr = gld16(vp + (int64_t)my_n * p.sv.s + ks * 16 + 8 * g);
+        for (int ks = 0; ks < C::KSTEPS; ks++) {
+            i32x4 v = {0, 0, 0, 0};
+            if (my_n < N) v = gld16(src + ks * 16 + 8 * g);
+            opreg[ks] = as_vec<T8>(v);
         }
-        kreg[ks] = as_vec<T8>(kr);
-        vreg[ks] = as_vec<T8>(vr);
     }
 
     // ---- K of all 128 keys as B operand of dQ = dS K: column d = 32*dq_db + l%32, k = key.
     // Staged once through LDS and gathered down the columns.  The NDQ = NSUB * DB blocks of dQ of
-    // a query block are dealt to the waves: wave w owns blocks w*BPW .. w*BPW+BPW-1, block index
+    // a query block are dealt to the S-waves: wave w owns blocks w*BPW .. w*BPW+BPW-1, block index
     // = (head-dim block) * NSUB + (query sub-block), so all blocks of a wave share one head-dim
     // block and therefore one set of K^T registers.
-    const int dq_first = wave * C::BPW;
+    const int dq_first = kb * C::BPW;
     const int dq_db = dq_first / NSUB;
-    const bool dq_active = dq_first < C::NDQ;
+    const bool dq_active = s_wave && dq_first < C::NDQ;
     T8 ktreg[BN / 16];
     {
         T* kt_lds = reinterpret_cast<T*>(smem);
@@ -180,87 +195,112 @@ __global__ __launch_bounds__(256, 1) void fa_bwd_kernel(const BwdParams p) {
             lds_write16(kt_lds + row * C::KTS + ch * 8, v);
         }
         __syncthreads();
+        if (s_wave) {
 #pragma unroll
-        for (int ks = 0; ks < BN / 16; ks++) {
-            // natural key order in the k slots: rows 16 ks + 8 g + {0..7}
-            const int s = lane & 15;
-            const int col = ((dq_active ? dq_db : 0) * 32 + ((lane >> 4) & 1) * 16 + (s & 3) * 4) & (D - 1);
-            const int row = ks * 16 + 8 * g + (s >> 2);
-            i16x4 lo = lds_read_tr4(kt_lds + row * C::KTS + col);
-            i16x4 hi = lds_read_tr4(kt_lds + (row + 4) * C::KTS + col);
-            typedef short i16x8 __attribute__((ext_vector_type(8)));
-            ktreg[ks] = __builtin_bit_cast(T8, (i16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+            for (int ks = 0; ks < BN / 16; ks++) {
+                // natural key order in the k slots: rows 16 ks + 8 g + {0..7}
+                const int s = lane & 15;
+                const int col = ((dq_active ? dq_db : 0) * 32 + ((lane >> 4) & 1) * 16 + (s & 3) * 4) & (D - 1);
+                const int row = ks * 16 + 8 * g + (s >> 2);
+                i16x4 lo = lds_read_tr4(kt_lds + row * C::KTS + col);
+                i16x4 hi = lds_read_tr4(kt_lds + (row + 4) * C::KTS + col);
+                typedef short i16x8 __attribute__((ext_vector_type(8)));
+                ktreg[ks] = __builtin_bit_cast(T8, (i16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+            }
         }
         __syncthreads();  // the staging area is reused by the loop's tiles
     }
 
-    f32x16 dv_acc[C::DB], dk_acc[C::DB];
+    // dV^T (S-wave) or dK^T (dP-wave) of this wave's 32 keys: rows = head dim, columns = keys
+    f32x16 acc[C::DB];
 #pragma unroll
     for (int db = 0; db < C::DB; db++)
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-            dv_acc[db][i] = 0.f;
-            dk_acc[db][i] = 0.f;
-        }
+        for (int i = 0; i < 16; i++) acc[db][i] = 0.f;
 
     const float qk_scale = p.sm_scale * kLog2e;
     const int n_mblocks = (M + BMI - 1) / BMI;
     // causal: query blocks that end above the first key of this tile see none of its keys
     const int mb_first = CAUSAL ? (n0 / BMI) : 0;
-
-    // 16-byte chunk (row, ch) of this wave's 32-key slice of a (B, H, M, N) bias-like tensor
     const bool bias_vec = BIAS != 0 && p.bias_vec;
     const bool dbias_vec = DBIAS && p.dbias_vec;
-    constexpr int EPC = C::ES > 0 ? 16 / C::ES : 8;  // elements per 16-byte chunk
 
     // blocks skipped by the causal schedule still owe zeros to dBias
-    if (DBIAS && CAUSAL) {
+    if (DBIAS && CAUSAL && !s_wave) {
         const int rows_skipped = mb_first * BMI < M ? mb_first * BMI : M;
         for (int c = lane; c < rows_skipped * C::BCPR; c += 64) {
-            const int m = c / C::BCPR, nn = nw + (c % C::BCPR) * EPC;
+            const int m = c / C::BCPR, nn = nw + (c % C::BCPR) * C::EPC;
             E* dst = dbp + (int64_t)m * p.sdbias.m + (int64_t)nn * p.sdbias.n;
-            if (dbias_vec && nn + EPC <= N) {
+            if (dbias_vec && nn + C::EPC <= N) {
                 i32x4 z = {0, 0, 0, 0};
                 gst16(dst, z);
             } else {
-                for (int e = 0; e < EPC; e++)
+                for (int e = 0; e < C::EPC; e++)
                     if (nn + e < N) dst[(int64_t)e * p.sdbias.n] = (E)0.f;
             }
         }
     }
 
-    i32x4 qreg[C::NCH], doreg[C::NCH];
-    i32x4 breg[C::BCH > 0 ? C::BCH : 1];
-    float lse_r = 0.f, delta_r = 0.f;
-    auto prefetch = [&](int mb) {
+    // ---- global -> register staging, one query block ahead --------------------------------
+    // Q / dO rows through buffer views of this (b, h) slice: rows past M read as zero.
+    const __amdgpu_buffer_rsrc_t q_rsrc = make_buffer(qp, ((int64_t)(M - 1) * p.sq.s + D) * 2);
+    const __amdgpu_buffer_rsrc_t do_rsrc = make_buffer(dop, ((int64_t)(M - 1) * p.sdo.s + D) * 2);
+    int q_off[C::QCH], do_off[C::QCH];
+#pragma unroll
+    for (int it = 0; it < C::QCH; it++) {
+        const int c = it * C::NT + tid;
+        q_off[it] = (c / CPR) * (int)p.sq.s * 2 + (c % CPR) * 16;
+        do_off[it] = (c / CPR) * (int)p.sdo.s * 2 + (c % CPR) * 16;
+    }
+    i32x4 qreg[C::QCH], doreg[C::QCH];
+    float stat_r = 0.f;
+    auto fetch_block = [&](int mb) {  // issue the loads of query block mb
         const int m0 = mb * BMI;
 #pragma unroll
-        for (int it = 0; it < C::NCH; it++) {
-            int c = it * C::NT + tid;
-            int row = c / CPR, ch = c % CPR;
-            bool ok = (c < BMI * CPR) && (m0 + row < M);
-            i32x4 z = {0, 0, 0, 0};
-            qreg[it] = ok ? gld16(qp + (int64_t)(m0 + row) * p.sq.s + ch * 8) : z;
-            doreg[it] = ok ? gld16(dop + (int64_t)(m0 + row) * p.sdo.s + ch * 8) : z;
+        for (int it = 0; it < C::QCH; it++) {
+            if (it * C::NT + (tid & ~63) < BMI * CPR) {  // wave-uniform
+                qreg[it] = buf_load16(q_rsrc, q_off[it], m0 * (int)p.sq.s * 2);
+                doreg[it] = buf_load16(do_rsrc, do_off[it], m0 * (int)p.sdo.s * 2);
+            }
         }
-        if (tid < BMI) {
-            lse_r = (m0 + tid < M) ? lsep[m0 + tid] : 0.f;
-            delta_r = (m0 + tid < M) ? deltap[m0 + tid] : 0.f;
+        if (tid < 2 * BMI) {
+            const int m = m0 + (tid & (BMI - 1));
+            const float* src = tid < BMI ? lsep : deltap;
+            stat_r = m < M ? src[m] : 0.f;
         }
+    };
+    auto stage_block = [&](int buf) {  // registers -> LDS tiles of buffer `buf`
+        T* q_lds = reinterpret_cast<T*>(smem + buf * C::Q_BYTES);
+        T* do_lds = reinterpret_cast<T*>(smem + C::OFF_DO + buf * C::Q_BYTES);
+#pragma unroll
+        for (int it = 0; it < C::QCH; it++) {
+            const int c = it * C::NT + tid;
+            if (c < BMI * CPR) {
+                lds_write16(q_lds + SW::off(c / CPR, (c % CPR) * 8), qreg[it]);
+                lds_write16(do_lds + SW::off(c / CPR, (c % CPR) * 8), doreg[it]);
+            }
+        }
+        if (tid < 2 * BMI) reinterpret_cast<float*>(smem + C::OFF_STAT + buf * C::STAT_BYTES)[tid] = stat_r;
+    };
+
+    // bias slice of an S-wave (BMI rows x 32 keys), one block ahead, through a buffer view
+    i32x4 breg[C::BCH > 0 ? C::BCH : 1];
+    auto fetch_bias = [&](int mb) {
         if constexpr (BIAS != 0) {
+            const int m0 = mb * BMI;
 #pragma unroll
             for (int it = 0; it < C::BCH; it++) {
                 const int c = it * 64 + lane;
-                const int m = m0 + c / C::BCPR, nn = nw + (c % C::BCPR) * EPC;
+                const int m = m0 + c / C::BCPR, nn = nw + (c % C::BCPR) * C::EPC;
                 const E* src = bp + (int64_t)m * p.sbias.m + (int64_t)nn * p.sbias.n;
                 i32x4 v = {0, 0, 0, 0};
-                if (m < M) {
-                    if (bias_vec && nn + EPC <= N) {
+                if (c < BMI * C::BCPR && m < M) {
+                    if (bias_vec && nn + C::EPC <= N) {
                         v = gld16(src);
                     } else {
-                        E tmp[EPC];
+                        E tmp[C::EPC];
 #pragma unroll
-                        for (int e = 0; e < EPC; e++) tmp[e] = (nn + e < N) ? src[(int64_t)e * p.sbias.n] : (E)0.f;
+                        for (int e = 0; e < C::EPC; e++) tmp[e] = (nn + e < N) ? src[(int64_t)e * p.sbias.n] : (E)0.f;
                         v = __builtin_bit_cast(i32x4, tmp);
                     }
                 }
@@ -268,206 +308,225 @@ __global__ __launch_bounds__(256, 1) void fa_bwd_kernel(const BwdParams p) {
             }
         }
     };
-    auto stage = [&](int buf) {  // registers -> LDS tiles of buffer `buf`
-        T* q_lds = reinterpret_cast<T*>(smem + buf * C::Q_BYTES);
-        T* do_lds = reinterpret_cast<T*>(smem + C::OFF_DO + buf * C::Q_BYTES);
-        float* st = reinterpret_cast<float*>(smem + C::OFF_STAT + buf * C::STAT_BYTES);
-#pragma unroll
-        for (int it = 0; it < C::NCH; it++) {
-            int c = it * C::NT + tid;
-            int row = c / CPR, ch = c % CPR;
-            if (c < BMI * CPR) {
-                lds_write16(q_lds + SW::off(row, ch * 8), qreg[it]);
-                lds_write16(do_lds + SW::off(row, ch * 8), doreg[it]);
-            }
-        }
-        if (tid < BMI) {
-            st[tid] = lse_r;
-            st[BMI + tid] = delta_r;
-        }
-    };
 
-    int buf = 0;
     if (mb_first < n_mblocks) {
-        prefetch(mb_first);
-        stage(0);
+        fetch_block(mb_first);
+        if (s_wave) fetch_bias(mb_first);
+        stage_block(mb_first & 1);
+        if (mb_first + 1 < n_mblocks) fetch_block(mb_first + 1);
     }
     __syncthreads();
 
-    for (int mb = mb_first; mb < n_mblocks; mb++, buf ^= 1) {
-        const int m0 = mb * BMI;
+    T8 opT[NSUB][2];  // P^T (S-wave) or dS^T (dP-wave) of the current block, packed as B operands
+    const __amdgpu_buffer_rsrc_t dq_rsrc = make_buffer(dqap, (int64_t)M * D * 4);
+
+    for (int t = mb_first; t <= n_mblocks; t++) {
+        const int buf = t & 1;
+        const bool live = t < n_mblocks;  // block t exists (the last step only drains block t - 1)
+        const bool prev = t > mb_first;   // block t - 1 exists
+        const int m0 = t * BMI;
         const T* q_lds = reinterpret_cast<const T*>(smem + buf * C::Q_BYTES);
         const T* do_lds = reinterpret_cast<const T*>(smem + C::OFF_DO + buf * C::Q_BYTES);
-        T* ds_lds = reinterpret_cast<T*>(smem + C::OFF_DS + buf * C::DS_BYTES);
-        const float* lse_lds = reinterpret_cast<const float*>(smem + C::OFF_STAT + buf * C::STAT_BYTES);
-        const float* delta_lds = lse_lds + BMI;
-
-        // this block's bias slice: registers -> wave-private LDS tile [BMI][32]
-        if constexpr (BIAS != 0) {
-#pragma unroll
-            for (int it = 0; it < C::BCH; it++) lds_write16(bt_lds + (it * 64 + lane) * 16, breg[it]);
-        }
-        if (mb + 1 < n_mblocks) prefetch(mb + 1);
-
+        const T* q_prev = reinterpret_cast<const T*>(smem + (buf ^ 1) * C::Q_BYTES);
+        T* ds_cur = reinterpret_cast<T*>(smem + C::OFF_DS + buf * C::DS_BYTES);
+        const T* ds_prev = reinterpret_cast<const T*>(smem + C::OFF_DS + (buf ^ 1) * C::DS_BYTES);
+        const float* stat_lds = reinterpret_cast<const float*>(smem + C::OFF_STAT + buf * C::STAT_BYTES);
         const bool need_mask = (m0 + BMI > M) || (n0 + BN > N) || (CAUSAL && m0 < n0 + BN - 1);
 
-        // ---- S = Q K^T and dP = dO V^T for both 32-row sub-blocks ----
-        f32x16 s[NSUB], dp[NSUB];
+        // =============================== first half ===============================
+        f32x16 sacc[NSUB];  // S (S-wave) or dP (dP-wave)
+        if (live) {
+            if constexpr (BIAS != 0) {
+                if (s_wave) {
+                    // this block's bias slice: registers -> wave-private LDS tile [BMI][32]
 #pragma unroll
-        for (int sb = 0; sb < NSUB; sb++) {
-#pragma unroll
-            for (int i = 0; i < 16; i++) {
-                s[sb][i] = 0.f;
-                dp[sb][i] = 0.f;
-            }
-#pragma unroll
-            for (int ks = 0; ks < C::KSTEPS; ks++) {
-                T8 a = as_vec<T8>(lds_read16(q_lds + SW::off(sb * 32 + r, ks * 16 + 8 * g)));
-                s[sb] = mfma32(a, kreg[ks], s[sb]);
-            }
-#pragma unroll
-            for (int ks = 0; ks < C::KSTEPS; ks++) {
-                T8 a = as_vec<T8>(lds_read16(do_lds + SW::off(sb * 32 + r, ks * 16 + 8 * g)));
-                dp[sb] = mfma32(a, vreg[ks], dp[sb]);
-            }
-        }
-
-        // ---- P and dS (flash_attention.py:281-306); register i of sub-block sb is row
-        // m0 + 32 sb + 8 (i/4) + 4 g + i%4, the lane is key my_n ----
-        T8 pT[NSUB][2], dsT[NSUB][2];
-#pragma unroll
-        for (int sb = 0; sb < NSUB; sb++) {
-#pragma unroll
-            for (int q4 = 0; q4 < 4; q4++) {
-                const int ml0 = sb * 32 + 8 * q4 + 4 * g;  // first of 4 consecutive rows
-                const f32x4 lse4 = *reinterpret_cast<const f32x4*>(lse_lds + ml0);
-                const f32x4 del4 = *reinterpret_cast<const f32x4*>(delta_lds + ml0);
-                float bv[4] = {0.f, 0.f, 0.f, 0.f};
-                if constexpr (BIAS == 1) {
-#pragma unroll
-                    for (int e = 0; e < 4; e++) bv[e] = bt_lds[(ml0 + e) * 32 + r] ? 0.f : kMask;
-                } else if constexpr (BIAS == 2 || BIAS == 3) {
-                    typedef typename VecOf<E>::v4 B4;
-                    i16x4 raw = lds_read_tr4(reinterpret_cast<const E*>(bt_lds) + tr_offset(lane, ml0, 0, 32));
-                    B4 hv = __builtin_bit_cast(B4, raw);
-#pragma unroll
-                    for (int e = 0; e < 4; e++) bv[e] = (float)hv[e] * kLog2e;
-                } else if constexpr (BIAS == 4) {
-#pragma unroll
-                    for (int e = 0; e < 4; e++) bv[e] = reinterpret_cast<const float*>(bt_lds)[(ml0 + e) * 32 + r] * kLog2e;
+                    for (int it = 0; it < C::BCH; it++)
+                        if (it * 64 + lane < BMI * C::BCPR) lds_write16(bt_lds + (it * 64 + lane) * 16, breg[it]);
+                    if (t + 1 < n_mblocks) fetch_bias(t + 1);
                 }
+            }
+            const T* a_tile = s_wave ? q_lds : do_lds;
 #pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const int i = q4 * 4 + e;
-                    const int m = m0 + ml0 + e;
-                    float x = __fmul_rn(s[sb][i], qk_scale);
-                    float add = bv[e];
-                    if (need_mask) {
-                        const bool oob = (m >= M) || (my_n >= N);
-                        float t = oob ? kMask : 0.f;
-                        if (CAUSAL) t += (m < my_n) ? kMask : 0.f;
-                        if (BIAS != 0) add = oob ? kMask : add;
-                        add = t + add;
-                    }
-                    x = __fadd_rn(x, add);
-                    const float pv = fast_exp2(x - lse4[e]);
-                    const float dsv = pv * (dp[sb][i] - del4[e]);
-                    pT[sb][i >> 3][i & 7] = (T)pv;
-                    dsT[sb][i >> 3][i & 7] = (T)dsv;
-                    ds_lds[(ml0 + e) * DSS + wave * 32 + r] = (T)dsv;
-                    if constexpr (DBIAS && !DB_VIA_LDS) {
-                        if (m < M && my_n < N) dbp[(int64_t)m * p.sdbias.m + (int64_t)my_n * p.sdbias.n] = (E)dsv;
-                    }
+            for (int sb = 0; sb < NSUB; sb++) {
+#pragma unroll
+                for (int i = 0; i < 16; i++) sacc[sb][i] = 0.f;
+#pragma unroll
+                for (int ks = 0; ks < C::KSTEPS; ks++) {
+                    T8 a = as_vec<T8>(lds_read16(a_tile + SW::off(sb * 32 + r, ks * 16 + 8 * g)));
+                    sacc[sb] = mfma32(a, opreg[ks], sacc[sb]);
                 }
             }
         }
-
-        // ---- dV^T += dO^T P and dK^T += Q^T dS ----
+        if (s_wave) {
+            if (live) {
+                // ---- P (flash_attention.py:281-294); register i of sub-block sb is row
+                // m0 + 32 sb + 8 (i/4) + 4 g + i%4, the lane is key my_n ----
 #pragma unroll
-        for (int sb = 0; sb < NSUB; sb++) {
+                for (int sb = 0; sb < NSUB; sb++) {
 #pragma unroll
-            for (int kk = 0; kk < 2; kk++) {
+                    for (int q4 = 0; q4 < 4; q4++) {
+                        const int ml0 = sb * 32 + 8 * q4 + 4 * g;  // first of 4 consecutive rows
+                        const f32x4 lse4 = *reinterpret_cast<const f32x4*>(stat_lds + ml0);
+                        float bv[4] = {0.f, 0.f, 0.f, 0.f};  // bias in log2 units / mask term
+                        if constexpr (BIAS == 1) {
 #pragma unroll
-                for (int db = 0; db < C::DB; db++) {
-                    T8 a = SW::template col8<T8>(do_lds, lane, sb * 32 + kk * 16, db * 32);
-                    dv_acc[db] = mfma32(a, pT[sb][kk], dv_acc[db]);
-                }
+                            for (int e = 0; e < 4; e++) bv[e] = bt_lds[(ml0 + e) * 32 + r] ? 0.f : kMask;
+                        } else if constexpr (BIAS == 2 || BIAS == 3) {
+                            typedef typename VecOf<E>::v4 B4;
+                            i16x4 raw = lds_read_tr4(reinterpret_cast<const E*>(bt_lds) + tr_offset(lane, ml0, 0, 32));
+                            B4 hv = __builtin_bit_cast(B4, raw);
 #pragma unroll
-                for (int db = 0; db < C::DB; db++) {
-                    T8 a = SW::template col8<T8>(q_lds, lane, sb * 32 + kk * 16, db * 32);
-                    dk_acc[db] = mfma32(a, dsT[sb][kk], dk_acc[db]);
-                }
-            }
-        }
-
-        // next block's tiles go into the other buffer while this one is still being read
-        if (mb + 1 < n_mblocks) stage(buf ^ 1);
-        __syncthreads();  // the dS tile of all 128 keys is complete; the next tiles are visible
-
-        // ---- dBias rows of this wave's 32 keys, 16 bytes per lane, out of the dS tile ----
-        if constexpr (DB_VIA_LDS) {
+                            for (int e = 0; e < 4; e++) bv[e] = (float)hv[e] * kLog2e;
+                        } else if constexpr (BIAS == 4) {
 #pragma unroll
-            for (int it = 0; it < (BMI * 4) / 64; it++) {
-                const int c = it * 64 + lane;
-                const int row = c >> 2, ch = c & 3;
-                const int m = m0 + row, nn = nw + ch * 8;
-                if (m < M && nn < N) {
-                    const T* src = ds_lds + row * DSS + wave * 32 + ch * 8;
-                    E* dst = dbp + (int64_t)m * p.sdbias.m + (int64_t)nn * p.sdbias.n;
-                    if (dbias_vec && nn + 8 <= N) {
-                        gst16(dst, lds_read16(src));
-                    } else {
-                        for (int e = 0; e < 8; e++)
-                            if (nn + e < N) dst[(int64_t)e * p.sdbias.n] = __builtin_bit_cast(E, src[e]);
+                            for (int e = 0; e < 4; e++)
+                                bv[e] = reinterpret_cast<const float*>(bt_lds)[(ml0 + e) * 32 + r] * kLog2e;
+                        }
+                        f32x4 p4;
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            const int i = q4 * 4 + e;
+                            float pv;
+                            if (need_mask) {
+                                const int m = m0 + ml0 + e;
+                                float x = __fmul_rn(sacc[sb][i], qk_scale);
+                                const bool oob = (m >= M) || (my_n >= N);
+                                float tmask = oob ? kMask : 0.f;
+                                if (CAUSAL) tmask += (m < my_n) ? kMask : 0.f;
+                                float add = bv[e];
+                                if (BIAS != 0) add = oob ? kMask : add;
+                                x = __fadd_rn(x, __fadd_rn(tmask, add));
+                                pv = fast_exp2(x - lse4[e]);
+                            } else {
+                                pv = fast_exp2(__builtin_fmaf(sacc[sb][i], qk_scale, bv[e] - lse4[e]));
+                            }
+                            p4[e] = pv;
+                            opT[sb][i >> 3][i & 7] = (T)pv;
+                        }
+                        // hand P to the dP-wave of the same keys: same lane, same register order
+                        *reinterpret_cast<f32x4*>(p_lds + ((sb * 4 + q4) * 64 + lane) * 4) = p4;
                     }
                 }
             }
+        } else if (prev) {
+            // ---- dK^T += Q^T dS of the previous block ----
+#pragma unroll
+            for (int sb = 0; sb < NSUB; sb++)
+#pragma unroll
+                for (int kk = 0; kk < 2; kk++)
+#pragma unroll
+                    for (int db = 0; db < C::DB; db++) {
+                        T8 a = SW::template col8<T8>(q_prev, lane, sb * 32 + kk * 16, db * 32);
+                        acc[db] = mfma32(a, opT[sb][kk], acc[db]);
+                    }
         }
+        __syncthreads();  // P(t) is visible to the dP-waves; nobody reads block t - 1's tiles any more
 
-        // ---- dQ blocks (32 rows x 32 head-dim columns each) += dS K ----
-        if (dq_active) {
+        // =============================== second half ===============================
+        if (t + 1 < n_mblocks) {
+            stage_block(buf ^ 1);                            // block t + 1 -> LDS
+            if (t + 2 < n_mblocks) fetch_block(t + 2);       // block t + 2 -> registers
+        }
+        if (s_wave) {
+            if (live) {
+                // ---- dV^T += dO^T P ----
 #pragma unroll
-            for (int j = 0; j < C::BPW; j++) {
-                const int sb = (dq_first + j) % NSUB;
-                f32x16 dq;
+                for (int sb = 0; sb < NSUB; sb++)
 #pragma unroll
-                for (int i = 0; i < 16; i++) dq[i] = 0.f;
+                    for (int kk = 0; kk < 2; kk++)
 #pragma unroll
-                for (int ks = 0; ks < BN / 16; ks++) {
-                    T8 a = as_vec<T8>(lds_read16(ds_lds + (sb * 32 + r) * DSS + ks * 16 + 8 * g));
-                    dq = mfma32(a, ktreg[ks], dq);
+                        for (int db = 0; db < C::DB; db++) {
+                            T8 a = SW::template col8<T8>(do_lds, lane, sb * 32 + kk * 16, db * 32);
+                            acc[db] = mfma32(a, opT[sb][kk], acc[db]);
+                        }
+            }
+            if (prev && dq_active) {
+                // ---- dQ blocks of the previous query block (32 rows x 32 head-dim columns each)
+                // += dS K over all 128 keys, added to the fp32 accumulator ----
+                const int mp = m0 - BMI;
+#pragma unroll
+                for (int j = 0; j < C::BPW; j++) {
+                    const int sb = (dq_first + j) % NSUB;
+                    f32x16 dq;
+#pragma unroll
+                    for (int i = 0; i < 16; i++) dq[i] = 0.f;
+#pragma unroll
+                    for (int ks = 0; ks < BN / 16; ks++) {
+                        T8 a = as_vec<T8>(lds_read16(ds_prev + (sb * 32 + r) * DSS + ks * 16 + 8 * g));
+                        dq = mfma32(a, ktreg[ks], dq);
+                    }
+                    const int d = dq_db * 32 + r;
+                    if (d < D) {
+                        const int voff = (4 * g * D + d) * 4;  // rows beyond M fall outside the view
+#pragma unroll
+                        for (int i = 0; i < 16; i++) {
+                            const int row = mp + sb * 32 + 8 * (i >> 2) + (i & 3);
+                            __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(dq[i], dq_rsrc, voff, row * D * 4, 0);
+                        }
+                    }
                 }
-                const int d = dq_db * 32 + r;
-                if (d < D) {
+            }
+        } else if (live) {
+            // ---- dS = P (dP - delta) (flash_attention.py:303-308) ----
+            const float* delta_lds = stat_lds + BMI;
 #pragma unroll
-                    for (int i = 0; i < 16; i++) {
-                        const int m = m0 + sb * 32 + 8 * (i >> 2) + 4 * g + (i & 3);
-                        if (m < M)
-                            __hip_atomic_fetch_add(dqap + (int64_t)m * D + d, dq[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for (int sb = 0; sb < NSUB; sb++) {
+#pragma unroll
+                for (int q4 = 0; q4 < 4; q4++) {
+                    const int ml0 = sb * 32 + 8 * q4 + 4 * g;
+                    const f32x4 del4 = *reinterpret_cast<const f32x4*>(delta_lds + ml0);
+                    const f32x4 p4 = *reinterpret_cast<const f32x4*>(p_lds + ((sb * 4 + q4) * 64 + lane) * 4);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const int i = q4 * 4 + e;
+                        const float dsv = p4[e] * (sacc[sb][i] - del4[e]);
+                        opT[sb][i >> 3][i & 7] = (T)dsv;
+                        ds_cur[(ml0 + e) * DSS + kb * 32 + r] = (T)dsv;
+                        if constexpr (DBIAS && !DB_VIA_LDS) {
+                            const int m = m0 + ml0 + e;
+                            if (m < M && my_n < N) dbp[(int64_t)m * p.sdbias.m + (int64_t)my_n * p.sdbias.n] = (E)dsv;
+                        }
+                    }
+                }
+            }
+            // ---- dBias rows of this wave's 32 keys, 16 bytes per lane, out of the dS tile ----
+            if constexpr (DB_VIA_LDS) {
+#pragma unroll
+                for (int it = 0; it < (BMI * 4) / 64; it++) {
+                    const int c = it * 64 + lane;
+                    const int row = c >> 2, ch = c & 3;
+                    const int m = m0 + row, nn = nw + ch * 8;
+                    if (m < M && nn < N) {
+                        const T* src = ds_cur + row * DSS + kb * 32 + ch * 8;
+                        E* dst = dbp + (int64_t)m * p.sdbias.m + (int64_t)nn * p.sdbias.n;
+                        if (dbias_vec && nn + 8 <= N) {
+                            gst16(dst, lds_read16(src));
+                        } else {
+                            for (int e = 0; e < 8; e++)
+                                if (nn + e < N) dst[(int64_t)e * p.sdbias.n] = __builtin_bit_cast(E, src[e]);
+                        }
                     }
                 }
             }
         }
+        __syncthreads();  // dS(t) and the tiles of block t + 1 are visible
     }
 
-    // ---- dK, dV of this wave's 32 keys (flash_attention.py:449-454) ----
+    // ---- dV (S-wave) or dK (dP-wave) of this wave's 32 keys (flash_attention.py:449-454) ----
     if (my_n < N) {
-        T* dkp = reinterpret_cast<T*>(p.dk) + (int64_t)b * p.sdk.b + (int64_t)h * p.sdk.h + (int64_t)my_n * p.sdk.s;
-        T* dvp = reinterpret_cast<T*>(p.dv) + (int64_t)b * p.sdv.b + (int64_t)h * p.sdv.h + (int64_t)my_n * p.sdv.s;
+        T* dst = s_wave ? reinterpret_cast<T*>(p.dv) + (int64_t)b * p.sdv.b + (int64_t)h * p.sdv.h + (int64_t)my_n * p.sdv.s
+                        : reinterpret_cast<T*>(p.dk) + (int64_t)b * p.sdk.b + (int64_t)h * p.sdk.h + (int64_t)my_n * p.sdk.s;
+        const float out_scale = s_wave ? 1.f : p.sm_scale;
 #pragma unroll
         for (int db = 0; db < C::DB; db++) {
 #pragma unroll
             for (int q4 = 0; q4 < 4; q4++) {
                 const int d = db * 32 + 8 * q4 + 4 * g;
                 if (d < D) {
-                    T4 kk4, vv4;
+                    T4 o4;
 #pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        kk4[e] = (T)(dk_acc[db][q4 * 4 + e] * p.sm_scale);
-                        vv4[e] = (T)dv_acc[db][q4 * 4 + e];
-                    }
-                    *reinterpret_cast<T4*>(dkp + d) = kk4;
-                    *reinterpret_cast<T4*>(dvp + d) = vv4;
+                    for (int e = 0; e < 4; e++) o4[e] = (T)(acc[db][q4 * 4 + e] * out_scale);
+                    *reinterpret_cast<T4*>(dst + d) = o4;
                 }
             }
         }
@@ -478,7 +537,7 @@ __global__ __launch_bounds__(256, 1) void fa_bwd_kernel(const BwdParams p) {
 template <typename T, int D, int BIAS, bool CAUSAL, bool DBIAS>
 static hipError_t launch_main(const BwdParams& p, hipStream_t st) {
     dim3 grid((unsigned)(p.n_ntiles * p.B * p.H));
-    hipLaunchKernelGGL((fa_bwd_kernel<T, D, BIAS, CAUSAL, DBIAS>), grid, dim3(256), 0, st, p);
+    hipLaunchKernelGGL((fa_bwd_kernel<T, D, BIAS, CAUSAL, DBIAS>), grid, dim3(512), 0, st, p);
     return hipGetLastError();
 }
 

@@ -94,8 +94,8 @@ const char *fa_strerror(int status);
  * Replaces _flash_attn_fwd, flash_attention.py:649-685 (bias pre-scale :660-663 included). */
 int fa_fwd(const fa_fwd_args *args, void *stream);
 
-/* Bytes of scratch the backward needs for this problem: delta (flash_attention.py:689) plus the
- * fp32 dQ accumulator.  Depends on B, H, M, D only. */
+/* Bytes of scratch the backward needs for this problem: delta, (B, H, M) fp32
+ * (flash_attention.py:689).  Depends on B, H, M only. */
 size_t fa_bwd_workspace_bytes(const fa_problem *p);
 
 /* Enqueue the backward (delta, dK/dV/dBias/dQ) on `stream`.
@@ -105,15 +105,15 @@ int fa_bwd(const fa_bwd_args *args, void *stream);
 /* The three stages fa_bwd enqueues, in order.  fa_bwd(args, stream) is
  * fa_bwd_stages(args, stream, FA_STAGE_ALL). */
 enum fa_bwd_stage {
-    FA_STAGE_PREP = 1, /* delta = rowsum(o * do) (flash_attention.py:197-233) + zero fill of the dQ accumulator */
-    FA_STAGE_MAIN = 2, /* dK, dV, dBias and the fp32 dQ accumulator (flash_attention.py:237-646) */
-    FA_STAGE_DQ = 4,   /* dq = accumulator * sm_scale in the output dtype (flash_attention.py:644-646) */
+    FA_STAGE_PREP = 1, /* delta = rowsum(o * do)          (flash_attention.py:197-233) */
+    FA_STAGE_MAIN = 2, /* dK, dV, dBias over key tiles    (flash_attention.py:237-454) */
+    FA_STAGE_DQ = 4,   /* dQ over query tiles              (flash_attention.py:458-646) */
     FA_STAGE_ALL = 7
 };
 
 /* Enqueue only the selected stages of the backward (same arguments and checks as fa_bwd).
  * No counterpart in the reference: it exists so that a benchmark or profiler can bracket one
- * stage with events; results are only meaningful after all three stages ran in order. */
+ * stage with events; FA_STAGE_MAIN and FA_STAGE_DQ both need the delta of FA_STAGE_PREP. */
 int fa_bwd_stages(const fa_bwd_args *args, void *stream, int stages);
 
 #ifdef __cplusplus

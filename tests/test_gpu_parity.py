@@ -102,13 +102,10 @@ def test_parity_causal(gpu_device, D, bias_kind):
         check(run_ours(q, k, v, do, bias, True), run_oracle(q, k, v, do, bias, True), "D%d %s S%d" % (D, bias_kind, S))
 
 
-def test_forward_head_dim_256(gpu_device):
-    for causal, bias_kind in ((False, None), (True, "bf16"), (False, "bool")):
-        q, k, v, do, bias = make_inputs(gpu_device, 1, 200, 200, 2, 256, torch.bfloat16, bias_kind, trainable=False)
-        with torch.no_grad():
-            out = flash_attention_fn(q, k, v, bias, causal)
-        ref = run_oracle(q, k, v, do, bias, causal)
-        assert (out.float() - ref["out"]).abs().max().item() <= OUT_ATOL
+def test_head_dim_256(gpu_device):
+    for causal, bias_kind in ((False, None), (True, "bf16"), (False, "bool"), (False, "f32")):
+        q, k, v, do, bias = make_inputs(gpu_device, 1, 200, 200, 2, 256, torch.bfloat16, bias_kind)
+        check(run_ours(q, k, v, do, bias, causal), run_oracle(q, k, v, do, bias, causal), "D256 %s" % bias_kind)
 
 
 def test_sm_scale_and_untrainable_bias(gpu_device):
@@ -208,7 +205,6 @@ def test_config5_cross_attention_alibi(gpu_device):
 
 # ---------------------------------------------------------------- exactness of masks
 def test_masked_keys_contribute_exactly_zero(gpu_device):
-    # one key tile (N <= 128): every output, dq included, has a single writer and is reproducible
     B, M, N, H, D = 2, 200, 120, 2, 64
     q, k, v, do, _ = make_inputs(gpu_device, B, M, N, H, D, torch.bfloat16, None, seed=21)
     mask = torch.ones(B, H, M, N, dtype=torch.bool, device=gpu_device)
@@ -223,7 +219,7 @@ def test_masked_keys_contribute_exactly_zero(gpu_device):
     assert torch.equal(a["dk"][:, :70], b["dk"][:, :70]) and torch.equal(a["dv"][:, :70], b["dv"][:, :70])
     assert (a["dk"][:, 70:] == 0).all() and (a["dv"][:, 70:] == 0).all()
     assert (b["dk"][:, 70:] == 0).all() and (b["dv"][:, 70:] == 0).all()
-    # several key tiles: out, dk, dv have single writers; dq is summed with atomics across key tiles
+    # several key tiles and a random key mask
     B, M, N, H, D = 1, 300, 700, 2, 128
     q, k, v, do, _ = make_inputs(gpu_device, B, M, N, H, D, torch.float16, None, seed=22)
     mask = (torch.rand(1, 1, 1, N, device=gpu_device) > 0.5).expand(B, H, M, N)
@@ -236,7 +232,7 @@ def test_masked_keys_contribute_exactly_zero(gpu_device):
     assert torch.equal(a["out"], b["out"])
     assert torch.equal(a["dk"][:, ~dead], b["dk"][:, ~dead]) and torch.equal(a["dv"][:, ~dead], b["dv"][:, ~dead])
     assert (a["dk"][:, dead] == 0).all() and (a["dv"][:, dead] == 0).all()
-    assert rel_l2(a["dq"], b["dq"]) < 1e-3
+    assert torch.equal(a["dq"], b["dq"])
 
 
 def test_fully_masked_rows_are_finite_and_match_oracle(gpu_device):
@@ -268,7 +264,7 @@ def test_causal_equals_lower_triangular_mask(gpu_device):
 
 # ---------------------------------------------------------------- layouts
 def test_packed_equals_unpacked_bit_for_bit(gpu_device):
-    B, S, H, D = 2, 128, 3, 64     # one key tile: dq has a single writer too
+    B, S, H, D = 2, 300, 3, 64
     g = torch.Generator().manual_seed(31)
     qkv = torch.randn(B, S, 3, H, D, generator=g).bfloat16().to(gpu_device).requires_grad_(True)
     do = torch.randn(B, S, H, D, generator=g).bfloat16().to(gpu_device)
@@ -296,6 +292,5 @@ def test_repeatability(gpu_device):
     q, k, v, do, bias = make_inputs(gpu_device, 1, 512, 512, 4, 128, torch.bfloat16, "bf16", seed=33)
     a = run_ours(q, k, v, do, bias, False)
     b = run_ours(q, k, v, do, bias, False)
-    for n in ("out", "dk", "dv", "dbias"):
-        assert torch.equal(a[n], b[n]), n
-    assert rel_l2(a["dq"], b["dq"]) < 1e-3      # fp32 atomics: order-dependent rounding only
+    for n in ("out", "dq", "dk", "dv", "dbias"):
+        assert torch.equal(a[n], b[n]), n           # every output element has a single writer

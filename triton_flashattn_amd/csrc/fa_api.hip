@@ -118,7 +118,7 @@ int fa_fwd(const fa_fwd_args* a, void* stream) {
 size_t fa_bwd_workspace_bytes(const fa_problem* p) {
     if (!p || check_problem(*p) != FA_OK) return 0;
     size_t rows = (size_t)p->B * p->H * p->M;
-    return align256(rows * sizeof(float)) + align256(rows * p->D * sizeof(float));
+    return align256(rows * sizeof(float));
 }
 
 int fa_bwd_stages(const fa_bwd_args* a, void* stream, int stages) {
@@ -142,9 +142,7 @@ int fa_bwd_stages(const fa_bwd_args* a, void* stream, int stages) {
     fa::BwdParams k{};
     k.q = a->q; k.k = a->k; k.v = a->v; k.o = a->o; k.dout = a->dout; k.bias = a->bias; k.lse = a->lse;
     k.dq = a->dq; k.dk = a->dk; k.dv = a->dv; k.dbias = a->dbias;
-    size_t rows = (size_t)p.B * p.H * p.M;
     k.delta = static_cast<float*>(a->workspace);
-    k.dq_acc = reinterpret_cast<float*>(static_cast<char*>(a->workspace) + align256(rows * sizeof(float)));
     k.sq = s3(a->q_strides); k.sk = s3(a->k_strides); k.sv = s3(a->v_strides); k.so = s3(a->o_strides);
     k.sdo = s3(a->do_strides); k.sdq = s3(a->dq_strides); k.sdk = s3(a->dk_strides); k.sdv = s3(a->dv_strides);
     if (a->bias) {
@@ -160,6 +158,7 @@ int fa_bwd_stages(const fa_bwd_args* a, void* stream, int stages) {
     int bn = fa::bwd_block_n(p.D);
     if (bn <= 0) return FA_ERR_UNSUPPORTED;
     k.n_ntiles = (p.N + bn - 1) / bn;
+    k.n_mtiles = (p.M + fa::fwd_block_m() - 1) / fa::fwd_block_m();
     hipError_t e = fa::launch_bwd(k, p.D, p.dtype, p.bias_dtype, p.causal != 0, a->dbias != nullptr, stages,
                                   static_cast<hipStream_t>(stream));
     if (e == hipErrorNotSupported) return FA_ERR_UNSUPPORTED;

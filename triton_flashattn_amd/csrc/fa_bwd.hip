@@ -1,28 +1,16 @@
-// Backward attention kernels for gfx950: dQ, dK, dV and dBias in a single pass over the score
-// matrix (5 matrix products per tile, bias read once, dBias written once).
+// Backward attention kernels for gfx950: dK, dV, dBias in one kernel over key tiles, dQ in a
+// second kernel over query tiles.  Every output element has exactly one writer, so results are
+// reproducible run to run, like the reference's (no atomics).
 //
 // Replaces _attn_bwd_preprocess, _attn_bwd_dkdv and _attn_bwd_dq of the reference
 // (/root/reference/flash_attention.py:197-646) and the host-side K / bias pre-scales
-// (flash_attention.py:699-704), which become fp32 multiplies inside the kernel.
+// (flash_attention.py:699-704), which become fp32 multiplies inside the kernels.
 //
-//   fa_bwd_prep_kernel     delta[b,h,m] = sum_d o * do  (flash_attention.py:215-227) and zero fill
-//                          of the fp32 dQ accumulator
-//   fa_bwd_kernel          one work-group (4 waves) owns 128 keys of one (batch, head); wave w owns
-//                          32 of them with K and V held in registers as B operands.  Query rows
-//                          are streamed in blocks of 64 (two 32-row sub-blocks) through
-//                          double-buffered LDS tiles.  Per sub-block:
-//                            S  = Q K^T, dP = dO V^T          (A = rows of Q / dO from LDS)
-//                            P  = 2^(S*scale + bias - LSE),  dS = P (dP - delta)
-//                            dV^T += dO^T P,  dK^T += Q^T dS  (A = columns of dO / Q gathered with
-//                                                              ds_read_b64_tr_b16, B = P / dS
-//                                                              straight from the accumulators)
-//                            dBias tile <- dS                  (flash_attention.py:307-308)
-//                            dS -> LDS, then dQ += dS K over all 128 keys, each wave one 32-wide
-//                            slice of the head dim, added to the fp32 accumulator with atomics
-//   fa_bwd_dq_kernel       dq = (T)(accumulator * sm_scale)   (flash_attention.py:644-646)
-//
-// In the accumulators a lane holds one key (column l%32) and 16 query rows, so bias loads and
-// dBias stores are contiguous across the lanes of a half-wave.
+//   fa_bwd_prep_kernel   delta[b,h,m] = sum_d o * do                  (flash_attention.py:215-227)
+//   fa_bwd_kernel        dK, dV, dBias of 128 keys per work-group     (flash_attention.py:237-454)
+//   fa_bwd_dq_kernel     dQ of 128 query rows per work-group          (flash_attention.py:458-646)
+#include <type_traits>
+
 #include "fa_common.hpp"
 #include "fa_params.hpp"
 
@@ -48,39 +36,301 @@ __global__ __launch_bounds__(256) void fa_bwd_prep_kernel(const BwdParams p) {
         T8 dv = as_vec<T8>(gld16(dp + c * 8));
 #pragma unroll
         for (int e = 0; e < 8; e++) acc += (float)ov[e] * (float)dv[e];
-        f32x4 z = {0.f, 0.f, 0.f, 0.f};
-        f32x4* za = reinterpret_cast<f32x4*>(p.dq_acc + row * D + c * 8);
-        za[0] = z;
-        za[1] = z;
     }
 #pragma unroll
     for (int w = LPR / 2; w >= 1; w >>= 1) acc += __shfl_xor(acc, w, 64);
     if (row < rows && c == 0) p.delta[row] = acc;
 }
 
-template <typename T, int D>
-__global__ __launch_bounds__(256) void fa_bwd_dq_kernel(const BwdParams p) {
-    constexpr int LPR = D / 8;
-    constexpr int RPB = 256 / LPR;
+// ---------------------------------------------------------------------------------------------
+// dQ kernel: a work-group owns 128 query rows (Q^T and dO^T in registers), streams K / V tiles
+// and recomputes S^T = K Q^T and dP^T = V dO^T, so that dS^T sits in the accumulator layout that
+// dQ^T += K^T dS^T wants as its B operand.  Replaces _attn_bwd_dq (flash_attention.py:458-646).
+template <typename T, int D, int BIAS, bool CAUSAL>
+__global__ __launch_bounds__(256, (RowCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_dq_kernel(const BwdParams p) {
+    typedef RowCfg<D, BIAS> C;
+    typedef Swz<D> SW;
     typedef typename VecOf<T>::v8 T8;
-    const int64_t rows = (int64_t)p.B * p.H * p.M;
-    const int64_t row = (int64_t)blockIdx.x * RPB + threadIdx.x / LPR;
-    const int c = threadIdx.x % LPR;
-    if (row >= rows) return;
-    const int m = (int)(row % p.M);
-    const int bh = (int)(row / p.M);
+    typedef typename VecOf<T>::v4 T4;
+    typedef typename BiasElem<BIAS>::type E;
+    constexpr int BM = C::BM, BN = C::BN, OS = C::OS, CPR = C::CPR;
+
+    __shared__ __align__(16) unsigned char smem[C::LDS_BYTES];
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int r = lane & 31, g = lane >> 5;
+
+    int mt, bh;
+    decode_block(blockIdx.x, p.n_mtiles, p.B * p.H, mt, bh);
+    if (CAUSAL) mt = p.n_mtiles - 1 - mt;  // longest rows first
     const int b = bh / p.H, h = bh % p.H;
-    const f32x4* src = reinterpret_cast<const f32x4*>(p.dq_acc + row * D + c * 8);
-    f32x4 lo = src[0], hi = src[1];
-    T8 out;
-#pragma unroll
-    for (int e = 0; e < 4; e++) {
-        out[e] = (T)(lo[e] * p.sm_scale);
-        out[4 + e] = (T)(hi[e] * p.sm_scale);
+    const int M = p.M, N = p.N;
+    const int m0 = mt * BM;
+    const int mw = m0 + wave * 32;  // first query row of this wave
+    const int my_m = mw + r;
+
+    const T* qp = reinterpret_cast<const T*>(p.q) + (int64_t)b * p.sq.b + (int64_t)h * p.sq.h;
+    const char* kbase = reinterpret_cast<const char*>(reinterpret_cast<const T*>(p.k) + (int64_t)b * p.sk.b + (int64_t)h * p.sk.h);
+    const char* vbase = reinterpret_cast<const char*>(reinterpret_cast<const T*>(p.v) + (int64_t)b * p.sv.b + (int64_t)h * p.sv.h);
+    const E* bp = nullptr;
+    unsigned char* bias_lds = nullptr;
+    if (BIAS != 0) {
+        bp = reinterpret_cast<const E*>(p.bias) + (int64_t)b * p.sbias.b + (int64_t)h * p.sbias.h;
+        bias_lds = smem + C::KV_BYTES + wave * 32 * C::BROW;
     }
-    T* dqp = reinterpret_cast<T*>(p.dq) + (int64_t)b * p.sdq.b + (int64_t)m * p.sdq.s + (int64_t)h * p.sdq.h;
-    gst16(dqp + c * 8, as_raw(out));
+
+    // Q^T and dO^T as B operands: column my_m, k = d
+    const T* dop = reinterpret_cast<const T*>(p.dout) + (int64_t)b * p.sdo.b + (int64_t)h * p.sdo.h;
+    T8 qreg[C::KSTEPS], doreg[C::KSTEPS];
+#pragma unroll
+    for (int ks = 0; ks < C::KSTEPS; ks++) {
+        i32x4 rq = {0, 0, 0, 0}, rd = {0, 0, 0, 0};
+        if (my_m < M) {
+            rq = gld16(qp + (int64_t)my_m * p.sq.s + ks * 16 + 8 * g);
+            rd = gld16(dop + (int64_t)my_m * p.sdo.s + ks * 16 + 8 * g);
+        }
+        qreg[ks] = as_vec<T8>(rq);
+        doreg[ks] = as_vec<T8>(rd);
+    }
+    // LSE (log2 units) and delta of this lane's query row
+    float lse_i = 0.f, delta_i = 0.f;
+    if (my_m < M) {
+        lse_i = p.lse[((int64_t)b * p.H + h) * M + my_m];
+        delta_i = p.delta[((int64_t)b * p.H + h) * M + my_m];
+    }
+
+    int n_tiles = (N + BN - 1) / BN;
+    if (CAUSAL) {
+        int last = (m0 + BM - 1) / BN + 1;  // tiles holding keys <= last row of this work-group
+        n_tiles = n_tiles < last ? n_tiles : last;
+    }
+
+    const float qk_scale = p.sm_scale * kLog2e;
+    f32x16 dq_acc[C::DB];  // dQ^T: rows = head dim, column = my_m
+#pragma unroll
+    for (int db = 0; db < C::DB; db++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) dq_acc[db][i] = 0.f;
+
+    // ---- K / V tiles: global -> LDS without passing through registers.  Chunk c of a tile
+    // (row c / CPR, LDS chunk c % CPR) is copied by thread c % 256 in copy c / 256; the LDS chunk
+    // holds global chunk (c % CPR) ^ f(row), which is the swizzle the readers expect.
+    unsigned koff[C::NCH], voff[C::NCH];  // byte offsets of this lane's source chunks in a full tile
+#pragma unroll
+    for (int it = 0; it < C::NCH; it++) {
+        const int c = it * C::NT + tid;
+        const int row = c / CPR, src = (c % CPR) ^ SW::f(row);
+        koff[it] = (unsigned)(row * (int)p.sk.s * 2 + src * 16);
+        voff[it] = (unsigned)(row * (int)p.sv.s * 2 + src * 16);
+    }
+    auto issue_tile = [&](int j, int buf) {
+        const int n0 = j * BN;
+        const char* kt = kbase + (int64_t)n0 * p.sk.s * 2;
+        const char* vt = vbase + (int64_t)n0 * p.sv.s * 2;
+        unsigned char* k_dst = smem + buf * C::TILE_BYTES;
+        unsigned char* v_dst = smem + (2 + buf) * C::TILE_BYTES;
+        const bool full = n0 + BN <= N;
+#pragma unroll
+        for (int it = 0; it < C::NCH; it++) {
+            const int c0 = it * C::NT + wave * 64;  // first chunk of this wave's copy
+            if (c0 < C::TILE_CHUNKS) {
+                unsigned ko = koff[it], vo = voff[it];
+                if (!full) {  // rows past the last key re-read the last key; the scores are masked
+                    const int c = c0 + lane;
+                    int row = c / CPR;
+                    const int src = (c % CPR) ^ SW::f(row);
+                    row = row < N - n0 ? row : N - n0 - 1;
+                    ko = (unsigned)(row * (int)p.sk.s * 2 + src * 16);
+                    vo = (unsigned)(row * (int)p.sv.s * 2 + src * 16);
+                }
+                g2lds16(kt + ko, k_dst + c0 * 16);
+                g2lds16(vt + vo, v_dst + c0 * 16);
+            }
+        }
+    };
+
+    // ---- bias tile of this wave (32 rows x 64 keys): global -> registers one tile ahead ----
+    i32x4 breg[C::BCH > 0 ? C::BCH : 1];
+    int boff[C::BCH > 0 ? C::BCH : 1];
+    __amdgpu_buffer_rsrc_t brsrc = make_buffer(nullptr, 0);
+    if constexpr (BIAS != 0) {
+        constexpr int CH_ROW = 4 * C::ES;  // 16-byte chunks per 64-key row
+#pragma unroll
+        for (int it = 0; it < C::BCH; it++) {
+            const int c = it * 64 + lane;
+            boff[it] = (c / CH_ROW) * (int)p.sbias.m * C::ES + (c % CH_ROW) * 16;
+        }
+        // everything from the first row of this wave to the end of the (b, h) slice
+        brsrc = make_buffer(bp + (int64_t)mw * p.sbias.m, ((int64_t)(M - 1 - mw) * p.sbias.m + N) * C::ES);
+    }
+    auto prefetch_bias = [&](int j) {
+        if constexpr (BIAS != 0) {
+            if (p.bias_vec) {
+#pragma unroll
+                for (int it = 0; it < C::BCH; it++) breg[it] = buf_load16(brsrc, boff[it], j * BN * C::ES);
+            }
+        }
+    };
+
+    if (n_tiles > 0) {
+        issue_tile(0, 0);
+        prefetch_bias(0);
+    }
+
+#pragma unroll 1
+    for (int j = 0; j < n_tiles; j++) {
+        const int n0 = j * BN;
+        const int buf = j & 1;
+        const T* k_lds = reinterpret_cast<const T*>(smem + buf * C::TILE_BYTES);
+        const T* v_lds = reinterpret_cast<const T*>(smem + (2 + buf) * C::TILE_BYTES);
+        __builtin_amdgcn_s_waitcnt(0);  // this thread's copies of tile j (and its bias chunks) have landed
+        if constexpr (BIAS != 0) {
+            if (p.bias_vec) {
+#pragma unroll
+                for (int it = 0; it < C::BCH; it++) {
+                    constexpr int CH_ROW = 4 * C::ES;
+                    const int c = it * 64 + lane;
+                    const int row = c / CH_ROW;
+                    lds_write16(bias_lds + row * C::BROW + (((c % CH_ROW) ^ C::bswz(row)) << 4), breg[it]);
+                }
+            } else {
+                // unaligned bias rows or non-unit key stride: one element per lane per row
+#pragma unroll 1
+                for (int row = 0; row < 32; row++) {
+                    int n = n0 + lane;
+                    E val = (E)0.f;
+                    if (mw + row < M && n < N)
+                        val = bp[(int64_t)(mw + row) * p.sbias.m + (int64_t)n * p.sbias.n];
+                    const int byte = lane * C::ES;
+                    *reinterpret_cast<E*>(bias_lds + row * C::BROW + (((byte >> 4) ^ C::bswz(row)) << 4) + (byte & 15)) = val;
+                }
+            }
+        }
+        __syncthreads();  // tile j is complete in LDS; nobody still reads the buffer of tile j - 1
+        if (j + 1 < n_tiles) {
+            issue_tile(j + 1, buf ^ 1);
+            prefetch_bias(j + 1);
+        }
+
+        // The 64-key tile is consumed as two 32-key halves, each with its own softmax step, so
+        // that only one 32 x 32 score block is live at a time.
+#pragma unroll
+        for (int nb = 0; nb < 2; nb++) {
+            const int nh = nb * 32;  // first key of this half inside the tile
+            __builtin_amdgcn_sched_barrier(0);  // keep the halves apart: one score block live at a time
+            // halves entirely above this wave's diagonal contribute nothing
+            if (CAUSAL && n0 + nh > mw + 31) continue;
+            if (n0 + nh >= N) continue;
+            const bool need_mask = (n0 + nh + 32 > N) || (CAUSAL && n0 + nh + 31 > mw);
+
+            // ---- S^T = K Q^T : s[i] is key n0 + nh + 8 (i/4) + 4 g + i%4, query my_m ----
+            f32x16 s;
+#pragma unroll
+            for (int i = 0; i < 16; i++) s[i] = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < C::KSTEPS; ks++) {
+                T8 a = as_vec<T8>(lds_read16(k_lds + SW::off(nh + r, ks * 16 + 8 * g)));
+                s = mfma32(a, qreg[ks], s);
+            }
+
+            // ---- dP^T = V dO^T ----
+            f32x16 dp;
+#pragma unroll
+            for (int i = 0; i < 16; i++) dp[i] = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < C::KSTEPS; ks++) {
+                T8 a = as_vec<T8>(lds_read16(v_lds + SW::off(nh + r, ks * 16 + 8 * g)));
+                dp = mfma32(a, doreg[ks], dp);
+            }
+
+            // ---- P = 2^(S*scale + bias - LSE), dS = P (dP - delta) (flash_attention.py:497-517).
+            // Masked tiles follow the reference's additive -1e6 arithmetic term by term.
+            T8 dsb[2];
+            auto ds_step = [&](auto masked_tag) {
+                constexpr bool MASKED = decltype(masked_tag)::value;
+#pragma unroll
+                for (int q4 = 0; q4 < 4; q4++) {
+                    const int nl = nh + 8 * q4 + 4 * g;  // first of 4 consecutive keys
+                    float bv[4] = {0.f, 0.f, 0.f, 0.f};  // bias in natural units
+                    bool keep[4] = {true, true, true, true};
+                    if constexpr (BIAS == 1) {
+                        unsigned int w = *reinterpret_cast<const unsigned int*>(bias_lds + r * C::BROW + (((nl >> 4) ^ C::bswz(r)) << 4) + (nl & 15));
+#pragma unroll
+                        for (int e = 0; e < 4; e++) keep[e] = ((w >> (8 * e)) & 0xffu) != 0;
+                    } else if constexpr (BIAS == 2 || BIAS == 3) {
+                        typedef typename VecOf<E>::v4 B4;
+                        B4 hv = *reinterpret_cast<const B4*>(bias_lds + r * C::BROW + (((nl >> 3) ^ C::bswz(r)) << 4) + ((nl * 2) & 15));
+#pragma unroll
+                        for (int e = 0; e < 4; e++) bv[e] = (float)hv[e];
+                    } else if constexpr (BIAS == 4) {
+                        f32x4 w = *reinterpret_cast<const f32x4*>(bias_lds + r * C::BROW + (((nl >> 2) ^ C::bswz(r)) << 4));
+#pragma unroll
+                        for (int e = 0; e < 4; e++) bv[e] = w[e];
+                    }
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const int i = q4 * 4 + e;
+                        float pv;
+                        if constexpr (MASKED) {
+                            float x = __fmul_rn(s[i], qk_scale);
+                            const int n = n0 + nl + e;
+                            const bool oob = (n >= N) || (my_m >= M);
+                            float t = oob ? kMask : 0.f;
+                            if (CAUSAL) t += (my_m < n) ? kMask : 0.f;
+                            float add = 0.f;
+                            if (BIAS == 1) add = keep[e] ? 0.f : kMask;
+                            if (BIAS >= 2) add = __fmul_rn(bv[e], kLog2e);
+                            if (BIAS != 0) add = oob ? kMask : add;  // out-of-range bias reads as masked
+                            x = __fadd_rn(x, __fadd_rn(t, add));
+                            pv = fast_exp2(x - lse_i);
+                        } else if constexpr (BIAS == 0) {
+                            pv = fast_exp2(__builtin_fmaf(s[i], qk_scale, -lse_i));
+                        } else if constexpr (BIAS == 1) {
+                            pv = fast_exp2(__builtin_fmaf(s[i], qk_scale, (keep[e] ? 0.f : kMask) - lse_i));
+                        } else {
+                            pv = fast_exp2(__builtin_fmaf(bv[e], kLog2e, __builtin_fmaf(s[i], qk_scale, -lse_i)));
+                        }
+                        dsb[i >> 3][i & 7] = (T)(pv * (dp[i] - delta_i));
+                    }
+                }
+            };
+            if (need_mask || m0 + BM > M) ds_step(std::true_type{});
+            else ds_step(std::false_type{});
+
+            // ---- dQ^T += K^T dS^T : A = K^T gathered down the columns of the K tile ----
+#pragma unroll
+            for (int kk = 0; kk < 2; kk++) {
+#pragma unroll
+                for (int db = 0; db < C::DB; db++) {
+                    T8 a = SW::template col8<T8>(k_lds, lane, nh + kk * 16, db * 32);
+                    dq_acc[db] = mfma32(a, dsb[kk], dq_acc[db]);
+                }
+            }
+        }
+    }
+
+    // ---- epilogue: dq = dQ * sm_scale (flash_attention.py:644-646) ----
+    __syncthreads();  // K/V tiles are dead: reuse their LDS for the output tile
+    T* o_lds = reinterpret_cast<T*>(smem) + wave * 32 * OS;
+#pragma unroll
+    for (int db = 0; db < C::DB; db++) {
+#pragma unroll
+        for (int q4 = 0; q4 < 4; q4++) {
+            T4 pk;
+#pragma unroll
+            for (int e = 0; e < 4; e++) pk[e] = (T)(dq_acc[db][q4 * 4 + e] * p.sm_scale);
+            *reinterpret_cast<T4*>(o_lds + r * OS + db * 32 + 8 * q4 + 4 * g) = pk;
+        }
+    }
+    __syncthreads();
+    T* op = reinterpret_cast<T*>(p.dq) + (int64_t)b * p.sdq.b + (int64_t)h * p.sdq.h;
+    for (int c = lane; c < 32 * CPR; c += 64) {
+        int row = c / CPR, ch = c % CPR;
+        if (mw + row < M) gst16(op + (int64_t)(mw + row) * p.sdq.s + ch * 8, lds_read16(o_lds + row * OS + ch * 8));
+    }
 }
+
 
 // ---------------------------------------------------------------------------------------------
 template <int D, int BIAS> struct BwdCfg {
@@ -93,7 +343,6 @@ template <int D, int BIAS> struct BwdCfg {
     static constexpr int CPR = D / 8;
     static constexpr int QCH = (BMI * CPR + NT - 1) / NT;  // 16-byte chunks per thread per Q (or dO) block
     static constexpr int DSS = BN + 8;                     // dS tile row stride (elements)
-    static constexpr int KTS = DP + 32;                    // one-time K tile (column gathers) row stride
     static constexpr int ES = BIAS == 0 ? 0 : (BIAS == 1 ? 1 : (BIAS == 4 ? 4 : 2));
     static constexpr int EPC = ES > 0 ? 16 / ES : 8;       // bias elements per 16-byte chunk
     static constexpr int BCPR = 2 * ES;                    // 16-byte chunks per 32-key bias row
@@ -109,21 +358,18 @@ template <int D, int BIAS> struct BwdCfg {
     static constexpr int OFF_STAT = OFF_P + P_BYTES;
     static constexpr int OFF_BIAS = OFF_STAT + 2 * STAT_BYTES;
     static constexpr int LOOP_BYTES = OFF_BIAS + 4 * BT_BYTES;
-    static constexpr int KT_BYTES = BN * KTS * 2;
-    static constexpr int LDS_BYTES = LOOP_BYTES > KT_BYTES ? LOOP_BYTES : KT_BYTES;
-    static constexpr int NDQ = NSUB * DB;                  // 32 x 32 blocks of dQ per query block
-    static constexpr int BPW = NDQ >= 4 ? NDQ / 4 : 1;     // dQ blocks per S-wave
+    static constexpr int LDS_BYTES = LOOP_BYTES;
 };
 
 // Work split inside a work-group of 8 waves.  Waves 0-3 ("S-waves") and waves 4-7 ("dP-waves")
 // pair up on the four 32-key blocks of the tile (waves w and w + 4 run on the same SIMD):
 //   S-wave : S = Q K^T, P = 2^(S*scale + bias - LSE)  -> hands P to its partner through LDS,
-//            dV^T += dO^T P, and one 32-wide head-dim slice of dQ += dS K (all 128 keys)
-//   dP-wave: dP = dO V^T, dS = P (dP - delta) -> dS tile in LDS (+ dBias), dK^T += Q^T dS
+//            dV^T += dO^T P
+//   dP-wave: dP = dO V^T, dS = P (dP - delta) (+ dBias through an LDS tile), dK^T += Q^T dS
 // A step handles one query block t and is cut in two by barriers so that in each half one wave
 // of a SIMD issues matrix instructions while the other does the exponentials / products:
 //   first half : S-wave: S(t), P(t)            dP-wave: dP(t), dK(t-1)
-//   second half: S-wave: dV(t), dQ(t-1)        dP-wave: dS(t), dBias(t)
+//   second half: S-wave: dV(t)                 dP-wave: dS(t), dBias(t)
 template <typename T, int D, int BIAS, bool CAUSAL, bool DBIAS>
 __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
     typedef BwdCfg<D, BIAS> C;
@@ -157,7 +403,6 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
     const T* dop = reinterpret_cast<const T*>(p.dout) + (int64_t)b * p.sdo.b + (int64_t)h * p.sdo.h;
     const float* lsep = p.lse + ((int64_t)b * p.H + h) * M;
     const float* deltap = p.delta + ((int64_t)b * p.H + h) * M;
-    float* dqap = p.dq_acc + ((int64_t)b * p.H + h) * M * D;
     const E* bp = nullptr;
     E* dbp = nullptr;
     if (BIAS != 0) bp = reinterpret_cast<const E*>(p.bias) + (int64_t)b * p.sbias.b + (int64_t)h * p.sbias.h;
@@ -175,40 +420,6 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
             if (my_n < N) v = gld16(src + ks * 16 + 8 * g);
             opreg[ks] = as_vec<T8>(v);
         }
-    }
-
-    // ---- K of all 128 keys as B operand of dQ = dS K: column d = 32*dq_db + l%32, k = key.
-    // Staged once through LDS and gathered down the columns.  The NDQ = NSUB * DB blocks of dQ of
-    // a query block are dealt to the S-waves: wave w owns blocks w*BPW .. w*BPW+BPW-1, block index
-    // = (head-dim block) * NSUB + (query sub-block), so all blocks of a wave share one head-dim
-    // block and therefore one set of K^T registers.
-    const int dq_first = kb * C::BPW;
-    const int dq_db = dq_first / NSUB;
-    const bool dq_active = s_wave && dq_first < C::NDQ;
-    T8 ktreg[BN / 16];
-    {
-        T* kt_lds = reinterpret_cast<T*>(smem);
-        for (int c = tid; c < BN * CPR; c += C::NT) {
-            int row = c / CPR, ch = c % CPR;
-            i32x4 v = {0, 0, 0, 0};
-            if (n0 + row < N) v = gld16(kp + (int64_t)(n0 + row) * p.sk.s + ch * 8);
-            lds_write16(kt_lds + row * C::KTS + ch * 8, v);
-        }
-        __syncthreads();
-        if (s_wave) {
-#pragma unroll
-            for (int ks = 0; ks < BN / 16; ks++) {
-                // natural key order in the k slots: rows 16 ks + 8 g + {0..7}
-                const int s = lane & 15;
-                const int col = ((dq_active ? dq_db : 0) * 32 + ((lane >> 4) & 1) * 16 + (s & 3) * 4) & (D - 1);
-                const int row = ks * 16 + 8 * g + (s >> 2);
-                i16x4 lo = lds_read_tr4(kt_lds + row * C::KTS + col);
-                i16x4 hi = lds_read_tr4(kt_lds + (row + 4) * C::KTS + col);
-                typedef short i16x8 __attribute__((ext_vector_type(8)));
-                ktreg[ks] = __builtin_bit_cast(T8, (i16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-            }
-        }
-        __syncthreads();  // the staging area is reused by the loop's tiles
     }
 
     // dV^T (S-wave) or dK^T (dP-wave) of this wave's 32 keys: rows = head dim, columns = keys
@@ -318,7 +529,6 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
     __syncthreads();
 
     T8 opT[NSUB][2];  // P^T (S-wave) or dS^T (dP-wave) of the current block, packed as B operands
-    const __amdgpu_buffer_rsrc_t dq_rsrc = make_buffer(dqap, (int64_t)M * D * 4);
 
     for (int t = mb_first; t <= n_mblocks; t++) {
         const int buf = t & 1;
@@ -329,7 +539,6 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
         const T* do_lds = reinterpret_cast<const T*>(smem + C::OFF_DO + buf * C::Q_BYTES);
         const T* q_prev = reinterpret_cast<const T*>(smem + (buf ^ 1) * C::Q_BYTES);
         T* ds_cur = reinterpret_cast<T*>(smem + C::OFF_DS + buf * C::DS_BYTES);
-        const T* ds_prev = reinterpret_cast<const T*>(smem + C::OFF_DS + (buf ^ 1) * C::DS_BYTES);
         const float* stat_lds = reinterpret_cast<const float*>(smem + C::OFF_STAT + buf * C::STAT_BYTES);
         const bool need_mask = (m0 + BMI > M) || (n0 + BN > N) || (CAUSAL && m0 < n0 + BN - 1);
 
@@ -440,32 +649,6 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
                             acc[db] = mfma32(a, opT[sb][kk], acc[db]);
                         }
             }
-            if (prev && dq_active) {
-                // ---- dQ blocks of the previous query block (32 rows x 32 head-dim columns each)
-                // += dS K over all 128 keys, added to the fp32 accumulator ----
-                const int mp = m0 - BMI;
-#pragma unroll
-                for (int j = 0; j < C::BPW; j++) {
-                    const int sb = (dq_first + j) % NSUB;
-                    f32x16 dq;
-#pragma unroll
-                    for (int i = 0; i < 16; i++) dq[i] = 0.f;
-#pragma unroll
-                    for (int ks = 0; ks < BN / 16; ks++) {
-                        T8 a = as_vec<T8>(lds_read16(ds_prev + (sb * 32 + r) * DSS + ks * 16 + 8 * g));
-                        dq = mfma32(a, ktreg[ks], dq);
-                    }
-                    const int d = dq_db * 32 + r;
-                    if (d < D) {
-                        const int voff = (4 * g * D + d) * 4;  // rows beyond M fall outside the view
-#pragma unroll
-                        for (int i = 0; i < 16; i++) {
-                            const int row = mp + sb * 32 + 8 * (i >> 2) + (i & 3);
-                            __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(dq[i], dq_rsrc, voff, row * D * 4, 0);
-                        }
-                    }
-                }
-            }
         } else if (live) {
             // ---- dS = P (dP - delta) (flash_attention.py:303-308) ----
             const float* delta_lds = stat_lds + BMI;
@@ -568,7 +751,21 @@ template <typename T, int D> static hipError_t launch_all(const BwdParams& p, in
         if (e != hipSuccess) return e;
     }
     if (stages & 4) {
-        hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D>), rgrid, dim3(256), 0, st, p);
+        dim3 qgrid((unsigned)(p.n_mtiles * p.B * p.H));
+#define FA_CASE(BK)                                                                                               \
+    case BK:                                                                                                      \
+        if (causal) hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, BK, true>), qgrid, dim3(256), 0, st, p);           \
+        else hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, BK, false>), qgrid, dim3(256), 0, st, p);                 \
+        break;
+        switch (bias) {
+            FA_CASE(0)
+            FA_CASE(1)
+            FA_CASE(2)
+            FA_CASE(3)
+            FA_CASE(4)
+            default: return hipErrorInvalidValue;
+        }
+#undef FA_CASE
         e = hipGetLastError();
     }
     return e;
@@ -580,6 +777,7 @@ template <typename T> static hipError_t launch_d(const BwdParams& p, int D, int 
         case 32: return launch_all<T, 32>(p, bias, causal, dbias, stages, st);
         case 64: return launch_all<T, 64>(p, bias, causal, dbias, stages, st);
         case 128: return launch_all<T, 128>(p, bias, causal, dbias, stages, st);
+        case 256: return launch_all<T, 256>(p, bias, causal, dbias, stages, st);
     }
     return hipErrorNotSupported;
 }
@@ -589,6 +787,6 @@ hipError_t launch_bwd(const BwdParams& p, int D, int dtype, int bias, bool causa
     return launch_d<__bf16>(p, D, bias, causal, dbias, stages, st);
 }
 
-int bwd_block_n(int D) { return D <= 128 ? 128 : 0; }
+int bwd_block_n(int) { return 128; }
 
 }  // namespace fa

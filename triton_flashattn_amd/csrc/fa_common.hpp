@@ -154,6 +154,33 @@ template <> struct BiasElem<2> { typedef _Float16 type; };
 template <> struct BiasElem<3> { typedef __bf16 type; };
 template <> struct BiasElem<4> { typedef float type; };
 
+// Tiling of the kernels in which a work-group owns 128 query rows (4 waves x 32 rows) and
+// streams keys in tiles of 64 through double-buffered LDS: the forward and the dQ kernel.
+template <int D, int BIAS> struct RowCfg {
+    static constexpr int BM = 128, BN = 64, NT = 256;
+    static constexpr int DP = D < 32 ? 32 : D;       // head dim padded to one 32-wide MFMA block
+    static constexpr int OS = DP + 8;                // O staging row stride (elements)
+    static constexpr int CPR = D / 8;                // 16-byte chunks per row
+    static constexpr int TILE_CHUNKS = BN * CPR;     // 16-byte chunks per K (or V) tile
+    static constexpr int NCH = (TILE_CHUNKS + NT - 1) / NT;  // direct-to-LDS copies per thread per tile
+    static constexpr int KSTEPS = D / 16;            // MFMA k-steps of Q K^T
+    static constexpr int DB = DP / 32;               // 32-wide blocks of the head dim
+    static constexpr int ES = BIAS == 0 ? 0 : (BIAS == 1 ? 1 : (BIAS == 4 ? 4 : 2));
+    static constexpr int BROW = 64 * ES;             // bias tile row: 64 keys, unpadded, chunk-swizzled
+    // 16-byte chunk c of bias row `row` is stored at chunk c ^ bswz(row)
+    __device__ static __forceinline__ int bswz(int row) {
+        return ES == 4 ? (row & 15) : (ES == 2 ? (row & 7) : ((row >> 2) & 3));
+    }
+    static constexpr int BCH = 2 * ES;               // 16-byte bias chunks per lane per tile
+    static constexpr int TILE_BYTES = BN * D * 2;    // unpadded, swizzled
+    static constexpr int O_BYTES = BM * OS * 2;
+    static constexpr int KV_BYTES = 4 * TILE_BYTES > O_BYTES ? 4 * TILE_BYTES : O_BYTES;  // K[2], V[2]
+    static constexpr int BIAS_BYTES = 4 * 32 * BROW;
+    static constexpr int LDS_BYTES = KV_BYTES + BIAS_BYTES;
+    // two work-groups per CU whenever registers allow it
+    static constexpr int MIN_BLOCKS = D <= 128 ? 2 : 1;
+};
+
 // Work-group id -> (tile, batch*head).  Work-groups are dealt round-robin to the 8 XCDs; when
 // the number of (batch, head) pairs is a multiple of 8 every tile of one pair is sent to the same
 // XCD so that its K/V (or Q/dO) stay in that XCD's L2.

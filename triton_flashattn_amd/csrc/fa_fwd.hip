@@ -21,34 +21,9 @@
 
 namespace fa {
 
-template <int D, int BIAS> struct FwdCfg {
-    static constexpr int BM = 128, BN = 64, NT = 256;
-    static constexpr int DP = D < 32 ? 32 : D;       // head dim padded to one 32-wide MFMA block
-    static constexpr int OS = DP + 8;                // O staging row stride (elements)
-    static constexpr int CPR = D / 8;                // 16-byte chunks per row
-    static constexpr int TILE_CHUNKS = BN * CPR;     // 16-byte chunks per K (or V) tile
-    static constexpr int NCH = (TILE_CHUNKS + NT - 1) / NT;  // direct-to-LDS copies per thread per tile
-    static constexpr int KSTEPS = D / 16;            // MFMA k-steps of Q K^T
-    static constexpr int DB = DP / 32;               // 32-wide blocks of the head dim
-    static constexpr int ES = BIAS == 0 ? 0 : (BIAS == 1 ? 1 : (BIAS == 4 ? 4 : 2));
-    static constexpr int BROW = 64 * ES;             // bias tile row: 64 keys, unpadded, chunk-swizzled
-    // 16-byte chunk c of bias row `row` is stored at chunk c ^ bswz(row)
-    __device__ static __forceinline__ int bswz(int row) {
-        return ES == 4 ? (row & 15) : (ES == 2 ? (row & 7) : ((row >> 2) & 3));
-    }
-    static constexpr int BCH = 2 * ES;               // 16-byte bias chunks per lane per tile
-    static constexpr int TILE_BYTES = BN * D * 2;    // unpadded, swizzled
-    static constexpr int O_BYTES = BM * OS * 2;
-    static constexpr int KV_BYTES = 4 * TILE_BYTES > O_BYTES ? 4 * TILE_BYTES : O_BYTES;  // K[2], V[2]
-    static constexpr int BIAS_BYTES = 4 * 32 * BROW;
-    static constexpr int LDS_BYTES = KV_BYTES + BIAS_BYTES;
-    // two work-groups per CU whenever registers allow it
-    static constexpr int MIN_BLOCKS = D <= 128 ? 2 : 1;
-};
-
 template <typename T, int D, int BIAS, bool CAUSAL>
-__global__ __launch_bounds__(256, (FwdCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_kernel(const FwdParams p) {
-    typedef FwdCfg<D, BIAS> C;
+__global__ __launch_bounds__(256, (RowCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_kernel(const FwdParams p) {
+    typedef RowCfg<D, BIAS> C;
     typedef Swz<D> SW;
     typedef typename VecOf<T>::v8 T8;
     typedef typename VecOf<T>::v4 T4;
@@ -236,26 +211,26 @@ __global__ __launch_bounds__(256, (FwdCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_ker
                 constexpr bool MASKED = decltype(masked_tag)::value;
                 float mx = -INFINITY;
                 {
-    #pragma unroll
+#pragma unroll
                     for (int q4 = 0; q4 < 4; q4++) {
                         const int nl = nh + 8 * q4 + 4 * g;  // first of 4 consecutive keys
                         float bv[4] = {0.f, 0.f, 0.f, 0.f};       // bias in natural units
                         bool keep[4] = {true, true, true, true};
                         if constexpr (BIAS == 1) {
                             unsigned int w = *reinterpret_cast<const unsigned int*>(bias_lds + r * C::BROW + (((nl >> 4) ^ C::bswz(r)) << 4) + (nl & 15));
-    #pragma unroll
+#pragma unroll
                             for (int e = 0; e < 4; e++) keep[e] = ((w >> (8 * e)) & 0xffu) != 0;
                         } else if constexpr (BIAS == 2 || BIAS == 3) {
                             typedef typename VecOf<E>::v4 B4;
                             B4 hv = *reinterpret_cast<const B4*>(bias_lds + r * C::BROW + (((nl >> 3) ^ C::bswz(r)) << 4) + ((nl * 2) & 15));
-    #pragma unroll
+#pragma unroll
                             for (int e = 0; e < 4; e++) bv[e] = (float)hv[e];
                         } else if constexpr (BIAS == 4) {
                             f32x4 w = *reinterpret_cast<const f32x4*>(bias_lds + r * C::BROW + (((nl >> 2) ^ C::bswz(r)) << 4));
-    #pragma unroll
+#pragma unroll
                             for (int e = 0; e < 4; e++) bv[e] = w[e];
                         }
-    #pragma unroll
+#pragma unroll
                         for (int e = 0; e < 4; e++) {
                             const int i = q4 * 4 + e;
                             float x;
@@ -292,14 +267,14 @@ __global__ __launch_bounds__(256, (FwdCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_ker
                     const float alpha = fast_exp2(m_i - m_new);
                     m_i = m_new;
                     l_i *= alpha;
-    #pragma unroll
+#pragma unroll
                     for (int db = 0; db < C::DB; db++)
-    #pragma unroll
+#pragma unroll
                         for (int i = 0; i < 16; i++) o_acc[db][i] *= alpha;
                 }
                 float rs = 0.f;
                 {
-    #pragma unroll
+#pragma unroll
                     for (int i = 0; i < 16; i++) {
                         float pv;
                         if constexpr (RAW || NAT) pv = fast_exp2(__builtin_fmaf(s[i], to_log2, -m_i));

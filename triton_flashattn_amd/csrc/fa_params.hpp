@@ -37,7 +37,6 @@ struct BwdParams {
     const void* bias;
     const float* lse;  // (B, H, M)
     float* delta;      // (B, H, M)        workspace
-    float* dq_acc;     // (B, H, M, D) fp32 workspace, zero on entry of the main kernel
     void* dq;
     void* dk;
     void* dv;
@@ -46,7 +45,8 @@ struct BwdParams {
     Strides4 sbias, sdbias;
     int B, H, M, N;
     float sm_scale;
-    int n_ntiles;
+    int n_ntiles;   // key tiles of the dK/dV kernel
+    int n_mtiles;   // query tiles of the dQ kernel
     int bias_vec;   // bias rows may be read with aligned 16-byte loads
     int dbias_vec;  // dbias rows may be written with aligned 16-byte stores
 };

@@ -89,7 +89,7 @@ class _HipBackend:
             _native.check(lib.fa_fwd(ctypes.byref(a), ctypes.c_void_p(stream)))
 
     def bwd_workspace(self, q, k, bias, causal, sm_scale):
-        """Scratch tensor of the size fa_bwd_workspace_bytes() asks for (delta + fp32 dQ accumulator)."""
+        """Scratch tensor of the size fa_bwd_workspace_bytes() asks for (delta)."""
         p = self._problem(q, k, bias, causal, sm_scale)
         nbytes = int(_native.load().fa_bwd_workspace_bytes(ctypes.byref(p)))
         if nbytes == 0:

@@ -7,8 +7,9 @@ bf16, B=2, H=16, M=N=4096, D=128, non-causal, trainable bf16 bias (B, H, M, N); 
 N(0, 1) tensors already resident in HBM.  Prints ONE JSON line on stdout (everything else goes to
 stderr).  Besides the whole-step throughput the line carries
 
-  roofline      the dominant kernel (the backward main kernel), timed with events on the launch
-                stream around the stage that runs only that kernel, against the HBM peak;
+  roofline      the dominant kernel (the backward kernel that produces dK, dV and dBias), timed
+                with events on the launch stream around the stage that runs only that kernel,
+                against the HBM peak;
   cpu_baseline  the eager fp32 oracle timed on this machine's host cores on a bounded sample;
   stages / other_configs   fwd, bwd and fwd+bwd of every BASELINE.json config.
 """
@@ -42,8 +43,8 @@ def algorithmic_bytes(B, H, M, N, D, causal, bias_es, trainable):
     lse = 4 * B * H * M
     y_fwd = q + 2 * kv + q + bias + lse
     y_bwd = (q + 2 * kv + q + q) + (q + 2 * kv) + lse + bias + (bias if trainable else 0)
-    # the backward main kernel alone: o is read by the delta stage only
-    y_main = y_bwd - q
+    # the dK/dV/dBias kernel alone: reads q, k, v, do, lse, delta, bias; writes dk, dv, dbias
+    y_main = (2 * q + 2 * kv) + 2 * kv + 2 * lse + bias + (bias if trainable else 0)
     return y_fwd, y_bwd, y_main, bias * (2 + (1 if trainable else 0))
 
 
@@ -94,7 +95,7 @@ def event_time_ms(fn, iters, warmup=2):
 
 
 def time_stages(cfg, iters):
-    """fwd, bwd (three stages), backward main kernel alone: milliseconds each."""
+    """fwd, bwd (three stages), dK/dV/dBias kernel alone, dQ kernel alone: milliseconds each."""
     import triton_flashattn_amd.flash_attention as fa
     from triton_flashattn_amd import _native
     q, k, v, do, bias, causal = cfg["q"], cfg["k"], cfg["v"], cfg["do"], cfg["bias"], cfg["causal"]
@@ -111,7 +112,8 @@ def time_stages(cfg, iters):
     t_bwd = event_time_ms(lambda: run(_native.FA_STAGE_ALL), iters)
     run(_native.FA_STAGE_PREP)
     t_main = event_time_ms(lambda: run(_native.FA_STAGE_MAIN), iters)
-    return t_fwd, t_bwd, t_main
+    t_dq = event_time_ms(lambda: run(_native.FA_STAGE_DQ), iters)
+    return t_fwd, t_bwd, t_main, t_dq
 
 
 def step(cfg):
@@ -173,6 +175,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-other-configs", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run one plain 1 GiB device-to-device copy and exit (reference point for "
+                         "the FETCH_SIZE / WRITE_SIZE counters of a profiler)")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this build runs on ONE GPU (every (batch, head) pair is independent, so more GPUs "
@@ -183,6 +188,14 @@ def main():
         sys.exit(3)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.calibrate_copy:
+        src = torch.ones(1 << 28, dtype=torch.float32, device=dev)   # 1 GiB
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        log("copied %d bytes" % (src.numel() * 4))
+        return
     from triton_flashattn_amd import _native
     _native.load()  # fail loudly before timing anything
 
@@ -202,8 +215,9 @@ def main():
     value = (f_fwd + f_bwd) / (ms_per_step * 1e-3) / 1e12
 
     iters = max(5, min(args.steps, 30))
-    t_fwd, t_bwd, t_main = time_stages(cfg, iters)
-    log("C3: step %.3f ms | fwd %.3f ms, bwd %.3f ms (main kernel %.3f ms)" % (ms_per_step, t_fwd, t_bwd, t_main))
+    t_fwd, t_bwd, t_main, t_dq = time_stages(cfg, iters)
+    log("C3: step %.3f ms | fwd %.3f ms, bwd %.3f ms (dK/dV/dBias kernel %.3f ms, dQ kernel %.3f ms)"
+        % (ms_per_step, t_fwd, t_bwd, t_main, t_dq))
     achieved = y_main / (t_main * 1e-3) / 1e9
     result = {
         "metric": "fwd+bwd TFLOP/s & bias HBM GB/s, bf16 B=2 H=16 M=N=4096 D=128",
@@ -218,7 +232,7 @@ def main():
         "hbm_roofline_frac_step": (y_fwd + y_bwd) / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "mfma_peak_frac_step": value / MFMA_PEAK_TFLOPS,
         "stages": {
-            "fwd_ms": t_fwd, "bwd_ms": t_bwd, "bwd_main_kernel_ms": t_main,
+            "fwd_ms": t_fwd, "bwd_ms": t_bwd, "bwd_dkdv_kernel_ms": t_main, "bwd_dq_kernel_ms": t_dq,
             "fwd_tflops": f_fwd / (t_fwd * 1e-3) / 1e12, "bwd_tflops": f_bwd / (t_bwd * 1e-3) / 1e12,
             "fwd_gbs": y_fwd / (t_fwd * 1e-3) / 1e9, "bwd_gbs": y_bwd / (t_bwd * 1e-3) / 1e9,
         },
@@ -227,7 +241,8 @@ def main():
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS, "traffic": None,
             "algorithmic_bytes_per_launch": y_main, "avg_launch_ms": t_main,
-            "mfma_frac_same_kernel": f_bwd / (t_main * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS,
+            # the kernel's own share of the algorithmic backward FLOPs: 4 of the 5 matrix products
+            "mfma_frac_same_kernel": 0.8 * f_bwd / (t_main * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS,
         },
         "peaks": {"hbm_gbs": HBM_PEAK_GBS, "mfma_bf16_tflops": MFMA_PEAK_TFLOPS},
     }
@@ -241,7 +256,7 @@ def main():
             Bc, Hc, Mc, Nc, Dc = cfg["dims"]
             ff, fb = flops(Bc, Hc, Mc, Nc, Dc, cfg["causal"])
             yf, yb, _, _ = algorithmic_bytes(Bc, Hc, Mc, Nc, Dc, cfg["causal"], cfg["bias_es"], cfg["trainable"])
-            tf, tb, tm = time_stages(cfg, 10)
+            tf, tb, tm, tq = time_stages(cfg, 10)
             others[name] = {
                 "fwd_ms": tf, "bwd_ms": tb, "fwd_bwd_ms": tf + tb,
                 "fwd_tflops": ff / (tf * 1e-3) / 1e12, "bwd_tflops": fb / (tb * 1e-3) / 1e12,

@@ -178,8 +178,10 @@ __global__ __launch_bounds__(256, (RowCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_dq_
         prefetch_bias(0);
     }
 
-#pragma unroll 1
-    for (int j = 0; j < n_tiles; j++) {
+    // One tile of the K/V stream.  Interior tiles (every key in range and visible to every row of
+    // the work-group) run with TILE_MASKED = false: no range checks, no mask arithmetic.
+    auto tile_step = [&](int j, auto tile_tag) {
+        constexpr bool TILE_MASKED = decltype(tile_tag)::value;
         const int n0 = j * BN;
         const int buf = j & 1;
         const T* k_lds = reinterpret_cast<const T*>(smem + buf * C::TILE_BYTES);
@@ -220,9 +222,9 @@ __global__ __launch_bounds__(256, (RowCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_dq_
             const int nh = nb * 32;  // first key of this half inside the tile
             __builtin_amdgcn_sched_barrier(0);  // keep the halves apart: one score block live at a time
             // halves entirely above this wave's diagonal contribute nothing
-            if (CAUSAL && n0 + nh > mw + 31) continue;
-            if (n0 + nh >= N) continue;
-            const bool need_mask = (n0 + nh + 32 > N) || (CAUSAL && n0 + nh + 31 > mw);
+            if (TILE_MASKED && CAUSAL && n0 + nh > mw + 31) continue;
+            if (TILE_MASKED && n0 + nh >= N) continue;
+            const bool need_mask = TILE_MASKED && ((n0 + nh + 32 > N) || (CAUSAL && n0 + nh + 31 > mw));
 
             // ---- S^T = K Q^T : s[i] is key n0 + nh + 8 (i/4) + 4 g + i%4, query my_m ----
             f32x16 s;
@@ -295,8 +297,12 @@ __global__ __launch_bounds__(256, (RowCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_dq_
                     }
                 }
             };
-            if (need_mask || m0 + BM > M) ds_step(std::true_type{});
-            else ds_step(std::false_type{});
+            if constexpr (TILE_MASKED) {
+                if (need_mask || m0 + BM > M) ds_step(std::true_type{});
+                else ds_step(std::false_type{});
+            } else {
+                ds_step(std::false_type{});
+            }
 
             // ---- dQ^T += K^T dS^T : A = K^T gathered down the columns of the K tile ----
 #pragma unroll
@@ -308,7 +314,16 @@ __global__ __launch_bounds__(256, (RowCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_dq_
                 }
             }
         }
-    }
+    };
+
+    int n_fast = N / BN;  // leading tiles that need no masks
+    if (CAUSAL) n_fast = n_fast < (m0 + 1) / BN ? n_fast : (m0 + 1) / BN;
+    if (n_fast > n_tiles) n_fast = n_tiles;
+    if (!(qk_scale > 0.f) || m0 + BM > M) n_fast = 0;
+#pragma unroll 1
+    for (int j = 0; j < n_fast; j++) tile_step(j, std::false_type{});
+#pragma unroll 1
+    for (int j = n_fast; j < n_tiles; j++) tile_step(j, std::true_type{});
 
     // ---- epilogue: dq = dQ * sm_scale (flash_attention.py:644-646) ----
     __syncthreads();  // K/V tiles are dead: reuse their LDS for the output tile

@@ -143,8 +143,10 @@ __global__ __launch_bounds__(256, (RowCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_ker
         prefetch_bias(0);
     }
 
-#pragma unroll 1
-    for (int j = 0; j < n_tiles; j++) {
+    // One tile of the K/V stream.  Interior tiles (every key in range and visible to every row of
+    // the work-group) run with TILE_MASKED = false: no range checks, no mask arithmetic.
+    auto tile_step = [&](int j, auto tile_tag) {
+        constexpr bool TILE_MASKED = decltype(tile_tag)::value;
         const int n0 = j * BN;
         const int buf = j & 1;
         const T* k_lds = reinterpret_cast<const T*>(smem + buf * C::TILE_BYTES);
@@ -185,9 +187,9 @@ __global__ __launch_bounds__(256, (RowCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_ker
             const int nh = nb * 32;  // first key of this half inside the tile
             __builtin_amdgcn_sched_barrier(0);  // keep the halves apart: one score block live at a time
             // halves entirely above this wave's diagonal contribute nothing
-            if (CAUSAL && n0 + nh > mw + 31) continue;
-            if (n0 + nh >= N) continue;
-            const bool need_mask = (n0 + nh + 32 > N) || (CAUSAL && n0 + nh + 31 > mw);
+            if (TILE_MASKED && CAUSAL && n0 + nh > mw + 31) continue;
+            if (TILE_MASKED && n0 + nh >= N) continue;
+            const bool need_mask = TILE_MASKED && ((n0 + nh + 32 > N) || (CAUSAL && n0 + nh + 31 > mw));
 
             // ---- S^T = K Q^T : s[i] is key n0 + nh + 8 (i/4) + 4 g + i%4, query my_m ----
             f32x16 s;
@@ -285,8 +287,12 @@ __global__ __launch_bounds__(256, (RowCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_ker
                 }
                 l_i += rs;  // per-lane partial sum; the two halves are added at the end
             };
-            if (need_mask || !(qk_scale > 0.f)) softmax_step(std::true_type{});
-            else softmax_step(std::false_type{});
+            if constexpr (TILE_MASKED) {
+                if (need_mask || !(qk_scale > 0.f)) softmax_step(std::true_type{});
+                else softmax_step(std::false_type{});
+            } else {
+                softmax_step(std::false_type{});
+            }
 
             // ---- O^T += V^T P^T : A = V^T gathered down the columns of the V tile ----
 #pragma unroll
@@ -298,7 +304,16 @@ __global__ __launch_bounds__(256, (RowCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_ker
                 }
             }
         }
-    }
+    };
+
+    int n_fast = N / BN;  // leading tiles that need no masks
+    if (CAUSAL) n_fast = n_fast < (m0 + 1) / BN ? n_fast : (m0 + 1) / BN;
+    if (n_fast > n_tiles) n_fast = n_tiles;
+    if (!(qk_scale > 0.f)) n_fast = 0;
+#pragma unroll 1
+    for (int j = 0; j < n_fast; j++) tile_step(j, std::false_type{});
+#pragma unroll 1
+    for (int j = n_fast; j < n_tiles; j++) tile_step(j, std::true_type{});
 
     // ---- epilogue (flash_attention.py:188-194) ----
     const float l_tot = pair_sum(l_i);

@@ -584,53 +584,60 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
         if (s_wave) {
             if (live) {
                 // ---- P (flash_attention.py:281-294); register i of sub-block sb is row
-                // m0 + 32 sb + 8 (i/4) + 4 g + i%4, the lane is key my_n ----
+                // m0 + 32 sb + 8 (i/4) + 4 g + i%4, the lane is key my_n.  Blocks that touch a ragged
+                // edge or the causal diagonal follow the reference's additive -1e6 arithmetic term by
+                // term; interior blocks fold everything into one exponent. ----
+                auto p_step = [&](auto masked_tag) {
+                    constexpr bool MASKED = decltype(masked_tag)::value;
 #pragma unroll
-                for (int sb = 0; sb < NSUB; sb++) {
+                    for (int sb = 0; sb < NSUB; sb++) {
 #pragma unroll
-                    for (int q4 = 0; q4 < 4; q4++) {
-                        const int ml0 = sb * 32 + 8 * q4 + 4 * g;  // first of 4 consecutive rows
-                        const f32x4 lse4 = *reinterpret_cast<const f32x4*>(stat_lds + ml0);
-                        float bv[4] = {0.f, 0.f, 0.f, 0.f};  // bias in log2 units / mask term
-                        if constexpr (BIAS == 1) {
+                        for (int q4 = 0; q4 < 4; q4++) {
+                            const int ml0 = sb * 32 + 8 * q4 + 4 * g;  // first of 4 consecutive rows
+                            const f32x4 lse4 = *reinterpret_cast<const f32x4*>(stat_lds + ml0);
+                            float bv[4] = {0.f, 0.f, 0.f, 0.f};  // bias in log2 units / mask term
+                            if constexpr (BIAS == 1) {
 #pragma unroll
-                            for (int e = 0; e < 4; e++) bv[e] = bt_lds[(ml0 + e) * 32 + r] ? 0.f : kMask;
-                        } else if constexpr (BIAS == 2 || BIAS == 3) {
-                            typedef typename VecOf<E>::v4 B4;
-                            i16x4 raw = lds_read_tr4(reinterpret_cast<const E*>(bt_lds) + tr_offset(lane, ml0, 0, 32));
-                            B4 hv = __builtin_bit_cast(B4, raw);
+                                for (int e = 0; e < 4; e++) bv[e] = bt_lds[(ml0 + e) * 32 + r] ? 0.f : kMask;
+                            } else if constexpr (BIAS == 2 || BIAS == 3) {
+                                typedef typename VecOf<E>::v4 B4;
+                                i16x4 raw = lds_read_tr4(reinterpret_cast<const E*>(bt_lds) + tr_offset(lane, ml0, 0, 32));
+                                B4 hv = __builtin_bit_cast(B4, raw);
 #pragma unroll
-                            for (int e = 0; e < 4; e++) bv[e] = (float)hv[e] * kLog2e;
-                        } else if constexpr (BIAS == 4) {
+                                for (int e = 0; e < 4; e++) bv[e] = (float)hv[e] * kLog2e;
+                            } else if constexpr (BIAS == 4) {
 #pragma unroll
-                            for (int e = 0; e < 4; e++)
-                                bv[e] = reinterpret_cast<const float*>(bt_lds)[(ml0 + e) * 32 + r] * kLog2e;
-                        }
-                        f32x4 p4;
-#pragma unroll
-                        for (int e = 0; e < 4; e++) {
-                            const int i = q4 * 4 + e;
-                            float pv;
-                            if (need_mask) {
-                                const int m = m0 + ml0 + e;
-                                float x = __fmul_rn(sacc[sb][i], qk_scale);
-                                const bool oob = (m >= M) || (my_n >= N);
-                                float tmask = oob ? kMask : 0.f;
-                                if (CAUSAL) tmask += (m < my_n) ? kMask : 0.f;
-                                float add = bv[e];
-                                if (BIAS != 0) add = oob ? kMask : add;
-                                x = __fadd_rn(x, __fadd_rn(tmask, add));
-                                pv = fast_exp2(x - lse4[e]);
-                            } else {
-                                pv = fast_exp2(__builtin_fmaf(sacc[sb][i], qk_scale, bv[e] - lse4[e]));
+                                for (int e = 0; e < 4; e++)
+                                    bv[e] = reinterpret_cast<const float*>(bt_lds)[(ml0 + e) * 32 + r] * kLog2e;
                             }
-                            p4[e] = pv;
-                            opT[sb][i >> 3][i & 7] = (T)pv;
+                            f32x4 p4;
+#pragma unroll
+                            for (int e = 0; e < 4; e++) {
+                                const int i = q4 * 4 + e;
+                                float pv;
+                                if constexpr (MASKED) {
+                                    const int m = m0 + ml0 + e;
+                                    float x = __fmul_rn(sacc[sb][i], qk_scale);
+                                    const bool oob = (m >= M) || (my_n >= N);
+                                    float tmask = oob ? kMask : 0.f;
+                                    if (CAUSAL) tmask += (m < my_n) ? kMask : 0.f;
+                                    float add = bv[e];
+                                    if (BIAS != 0) add = oob ? kMask : add;
+                                    x = __fadd_rn(x, __fadd_rn(tmask, add));
+                                    pv = fast_exp2(x - lse4[e]);
+                                } else {
+                                    pv = fast_exp2(__builtin_fmaf(sacc[sb][i], qk_scale, bv[e] - lse4[e]));
+                                }
+                                p4[e] = pv;
+                                opT[sb][i >> 3][i & 7] = (T)pv;
+                            }
+                            // hand P to the dP-wave of the same keys: same lane, same register order
+                            *reinterpret_cast<f32x4*>(p_lds + ((sb * 4 + q4) * 64 + lane) * 4) = p4;
                         }
-                        // hand P to the dP-wave of the same keys: same lane, same register order
-                        *reinterpret_cast<f32x4*>(p_lds + ((sb * 4 + q4) * 64 + lane) * 4) = p4;
                     }
-                }
+                };
+                if (need_mask) p_step(std::true_type{});
+                else p_step(std::false_type{});
             }
         } else if (prev) {
             // ---- dK^T += Q^T dS of the previous block ----

@@ -350,13 +350,13 @@ __global__ __launch_bounds__(256, (RowCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_dq_
 // ---------------------------------------------------------------------------------------------
 template <int D, int BIAS> struct BwdCfg {
     static constexpr int BN = 128, NT = 512;
-    static constexpr int NSUB = D <= 64 ? 2 : 1;     // 32-row sub-blocks of a query block
+    static constexpr int NSUB = (D <= 64 && BIAS != 4) ? 2 : 1;  // 32-row sub-blocks of a query block
     static constexpr int BMI = 32 * NSUB;
     static constexpr int DP = D < 32 ? 32 : D;
     static constexpr int DB = DP / 32;
     static constexpr int KSTEPS = D / 16;
     static constexpr int CPR = D / 8;
-    static constexpr int QCH = (BMI * CPR + NT - 1) / NT;  // 16-byte chunks per thread per Q (or dO) block
+    static constexpr int QCH = (BMI * CPR + 255) / 256;    // 16-byte chunks per dP-wave thread per Q (or dO) block
     static constexpr int DSS = BN + 8;                     // dS tile row stride (elements)
     static constexpr int ES = BIAS == 0 ? 0 : (BIAS == 1 ? 1 : (BIAS == 4 ? 4 : 2));
     static constexpr int EPC = ES > 0 ? 16 / ES : 8;       // bias elements per 16-byte chunk
@@ -372,7 +372,12 @@ template <int D, int BIAS> struct BwdCfg {
     static constexpr int OFF_P = OFF_DS + 2 * DS_BYTES;
     static constexpr int OFF_STAT = OFF_P + P_BYTES;
     static constexpr int OFF_BIAS = OFF_STAT + 2 * STAT_BYTES;
-    static constexpr int LOOP_BYTES = OFF_BIAS + 4 * BT_BYTES;
+    // The bias slices of an S-wave arrive through a ring of RING LDS slots filled by direct
+    // global -> LDS copies issued RING - 1 query blocks ahead: the bias is a pure HBM stream, and
+    // only a deep queue keeps enough bytes in flight to cover the memory latency.
+    static constexpr int RING_FIT = BT_BYTES > 0 ? (163840 - OFF_BIAS) / (4 * BT_BYTES) : 0;
+    static constexpr int RING = RING_FIT >= 8 ? 8 : (RING_FIT >= 4 ? 4 : 2);
+    static constexpr int LOOP_BYTES = OFF_BIAS + 4 * RING * BT_BYTES;
     static constexpr int LDS_BYTES = LOOP_BYTES;
 };
 
@@ -422,7 +427,7 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
     E* dbp = nullptr;
     if (BIAS != 0) bp = reinterpret_cast<const E*>(p.bias) + (int64_t)b * p.sbias.b + (int64_t)h * p.sbias.h;
     if (DBIAS) dbp = reinterpret_cast<E*>(p.dbias) + (int64_t)b * p.sdbias.b + (int64_t)h * p.sdbias.h;
-    unsigned char* bt_lds = smem + C::OFF_BIAS + kb * C::BT_BYTES;
+    unsigned char* ring_lds = smem + C::OFF_BIAS + kb * C::RING * C::BT_BYTES;
     float* p_lds = reinterpret_cast<float*>(smem + C::OFF_P) + kb * NSUB * 64 * 16;
 
     // ---- this wave's 32 keys as B operand (column my_n, k = d): K for an S-wave, V for a dP-wave
@@ -471,75 +476,92 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
     // Q / dO rows through buffer views of this (b, h) slice: rows past M read as zero.
     const __amdgpu_buffer_rsrc_t q_rsrc = make_buffer(qp, ((int64_t)(M - 1) * p.sq.s + D) * 2);
     const __amdgpu_buffer_rsrc_t do_rsrc = make_buffer(dop, ((int64_t)(M - 1) * p.sdo.s + D) * 2);
+    // Only the dP-waves fetch tiles (and the LSE / delta rows): the S-waves keep their
+    // vector-memory queue for the deep bias prefetch, whose completion is counted in order.
+    const int ftid = tid - 256;  // thread index among the dP-waves
     int q_off[C::QCH], do_off[C::QCH];
 #pragma unroll
     for (int it = 0; it < C::QCH; it++) {
-        const int c = it * C::NT + tid;
+        const int c = it * 256 + (ftid & 255);
         q_off[it] = (c / CPR) * (int)p.sq.s * 2 + (c % CPR) * 16;
         do_off[it] = (c / CPR) * (int)p.sdo.s * 2 + (c % CPR) * 16;
     }
     i32x4 qreg[C::QCH], doreg[C::QCH];
     float stat_r = 0.f;
-    auto fetch_block = [&](int mb) {  // issue the loads of query block mb
+    auto fetch_block = [&](int mb) {  // issue the loads of query block mb (dP-waves)
+        if (s_wave) return;
         const int m0 = mb * BMI;
 #pragma unroll
         for (int it = 0; it < C::QCH; it++) {
-            if (it * C::NT + (tid & ~63) < BMI * CPR) {  // wave-uniform
+            if (it * 256 + (ftid & ~63) < BMI * CPR) {  // wave-uniform
                 qreg[it] = buf_load16(q_rsrc, q_off[it], m0 * (int)p.sq.s * 2);
                 doreg[it] = buf_load16(do_rsrc, do_off[it], m0 * (int)p.sdo.s * 2);
             }
         }
-        if (tid < 2 * BMI) {
-            const int m = m0 + (tid & (BMI - 1));
-            const float* src = tid < BMI ? lsep : deltap;
+        if (ftid < 2 * BMI) {
+            const int m = m0 + (ftid & (BMI - 1));
+            const float* src = ftid < BMI ? lsep : deltap;
             stat_r = m < M ? src[m] : 0.f;
         }
     };
-    auto stage_block = [&](int buf) {  // registers -> LDS tiles of buffer `buf`
+    auto stage_block = [&](int buf) {  // registers -> LDS tiles of buffer `buf` (dP-waves)
+        if (s_wave) return;
         T* q_lds = reinterpret_cast<T*>(smem + buf * C::Q_BYTES);
         T* do_lds = reinterpret_cast<T*>(smem + C::OFF_DO + buf * C::Q_BYTES);
 #pragma unroll
         for (int it = 0; it < C::QCH; it++) {
-            const int c = it * C::NT + tid;
+            const int c = it * 256 + ftid;
             if (c < BMI * CPR) {
                 lds_write16(q_lds + SW::off(c / CPR, (c % CPR) * 8), qreg[it]);
                 lds_write16(do_lds + SW::off(c / CPR, (c % CPR) * 8), doreg[it]);
             }
         }
-        if (tid < 2 * BMI) reinterpret_cast<float*>(smem + C::OFF_STAT + buf * C::STAT_BYTES)[tid] = stat_r;
+        if (ftid < 2 * BMI) reinterpret_cast<float*>(smem + C::OFF_STAT + buf * C::STAT_BYTES)[ftid] = stat_r;
     };
 
-    // bias slice of an S-wave (BMI rows x 32 keys), one block ahead, through a buffer view
-    i32x4 breg[C::BCH > 0 ? C::BCH : 1];
-    auto fetch_bias = [&](int mb) {
+    // bias slice (BMI rows x 32 keys) of query block mb -> ring slot, straight from HBM to LDS.
+    // Chunk c = 64 it + lane of the slice (row c / BCPR, 16-byte chunk c % BCPR) lands at byte
+    // 16 c of the slot, i.e. the slot is the row-major slice.  Rows past M re-read row M - 1 and
+    // chunks that start past N re-read column 0: both are masked where they are used.  A block
+    // index past the end re-reads the last block, so that every step issues the same number of
+    // copies and their completion can be counted.
+    auto issue_bias = [&](int mb) {
         if constexpr (BIAS != 0) {
-            const int m0 = mb * BMI;
+            const int blk = mb < n_mblocks ? mb : n_mblocks - 1;
+            unsigned char* dst = ring_lds + ((mb - mb_first) & (C::RING - 1)) * C::BT_BYTES;
 #pragma unroll
             for (int it = 0; it < C::BCH; it++) {
                 const int c = it * 64 + lane;
-                const int m = m0 + c / C::BCPR, nn = nw + (c % C::BCPR) * C::EPC;
-                const E* src = bp + (int64_t)m * p.sbias.m + (int64_t)nn * p.sbias.n;
-                i32x4 v = {0, 0, 0, 0};
-                if (c < BMI * C::BCPR && m < M) {
-                    if (bias_vec && nn + C::EPC <= N) {
-                        v = gld16(src);
-                    } else {
-                        E tmp[C::EPC];
-#pragma unroll
-                        for (int e = 0; e < C::EPC; e++) tmp[e] = (nn + e < N) ? src[(int64_t)e * p.sbias.n] : (E)0.f;
-                        v = __builtin_bit_cast(i32x4, tmp);
-                    }
-                }
-                breg[it] = v;
+                int m = blk * BMI + c / C::BCPR;
+                int nn = nw + (c % C::BCPR) * C::EPC;
+                m = m < M ? m : M - 1;
+                nn = nn < N ? nn : 0;
+                g2lds16(bp + (int64_t)m * p.sbias.m + nn, dst + it * 1024);
+            }
+        }
+    };
+    // per-element path for bias rows that cannot be copied in aligned 16-byte chunks
+    auto load_bias_scalar = [&](int mb, unsigned char* dst) {
+        if constexpr (BIAS != 0) {
+            const int m0 = mb * BMI;
+#pragma unroll 1
+            for (int row = g; row < BMI; row += 2) {
+                const int m = m0 + row;
+                E val = (E)0.f;
+                if (m < M && my_n < N) val = bp[(int64_t)m * p.sbias.m + (int64_t)my_n * p.sbias.n];
+                reinterpret_cast<E*>(dst)[row * 32 + r] = val;
             }
         }
     };
 
     if (mb_first < n_mblocks) {
         fetch_block(mb_first);
-        if (s_wave) fetch_bias(mb_first);
         stage_block(mb_first & 1);
         if (mb_first + 1 < n_mblocks) fetch_block(mb_first + 1);
+        if (BIAS != 0 && s_wave && bias_vec) {
+#pragma unroll 1
+            for (int mb = mb_first; mb < mb_first + C::RING - 1; mb++) issue_bias(mb);
+        }
     }
     __syncthreads();
 
@@ -556,17 +578,22 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
         T* ds_cur = reinterpret_cast<T*>(smem + C::OFF_DS + buf * C::DS_BYTES);
         const float* stat_lds = reinterpret_cast<const float*>(smem + C::OFF_STAT + buf * C::STAT_BYTES);
         const bool need_mask = (m0 + BMI > M) || (n0 + BN > N) || (CAUSAL && m0 < n0 + BN - 1);
+        const unsigned char* bt_lds = ring_lds + ((t - mb_first) & (C::RING - 1)) * C::BT_BYTES;
 
         // =============================== first half ===============================
         f32x16 sacc[NSUB];  // S (S-wave) or dP (dP-wave)
         if (live) {
             if constexpr (BIAS != 0) {
                 if (s_wave) {
-                    // this block's bias slice: registers -> wave-private LDS tile [BMI][32]
-#pragma unroll
-                    for (int it = 0; it < C::BCH; it++)
-                        if (it * 64 + lane < BMI * C::BCPR) lds_write16(bt_lds + (it * 64 + lane) * 16, breg[it]);
-                    if (t + 1 < n_mblocks) fetch_bias(t + 1);
+                    if (bias_vec) {
+                        // the copies of block t were issued RING - 1 steps ago and at most the
+                        // (RING - 2) * BCH copies issued since may still be in flight
+                        constexpr int K = (C::RING - 2) * C::BCH;
+                        __builtin_amdgcn_s_waitcnt((K & 15) | ((K >> 4) << 14) | (7 << 4) | (15 << 8));
+                        issue_bias(t + C::RING - 1);  // into the slot block t - 1 has just left
+                    } else {
+                        load_bias_scalar(t, ring_lds + ((t - mb_first) & (C::RING - 1)) * C::BT_BYTES);
+                    }
                 }
             }
             const T* a_tile = s_wave ? q_lds : do_lds;

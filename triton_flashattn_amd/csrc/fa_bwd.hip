@@ -536,7 +536,7 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
                 int nn = nw + (c % C::BCPR) * C::EPC;
                 m = m < M ? m : M - 1;
                 nn = nn < N ? nn : 0;
-                g2lds16(bp + (int64_t)m * p.sbias.m + nn, dst + it * 1024);
+                g2lds16_untracked(bp + (int64_t)m * p.sbias.m + nn, dst + it * 1024);
             }
         }
     };
@@ -567,7 +567,11 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
 
     T8 opT[NSUB][2];  // P^T (S-wave) or dS^T (dP-wave) of the current block, packed as B operands
 
-    for (int t = mb_first; t <= n_mblocks; t++) {
+    // One step of the pipeline for one role.  The two roles run separate instances of the loop
+    // (same number of barriers each), so that the compiler's memory-wait bookkeeping of one role
+    // (tile loads counted by the compiler) never leaks into the other (bias copies counted by hand).
+    auto step = [&](int t, auto role_tag) {
+        constexpr bool IS_S = decltype(role_tag)::value;
         const int buf = t & 1;
         const bool live = t < n_mblocks;  // block t exists (the last step only drains block t - 1)
         const bool prev = t > mb_first;   // block t - 1 exists
@@ -583,20 +587,19 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
         // =============================== first half ===============================
         f32x16 sacc[NSUB];  // S (S-wave) or dP (dP-wave)
         if (live) {
-            if constexpr (BIAS != 0) {
-                if (s_wave) {
+            if constexpr (BIAS != 0 && IS_S) {
+                {
                     if (bias_vec) {
                         // the copies of block t were issued RING - 1 steps ago and at most the
                         // (RING - 2) * BCH copies issued since may still be in flight
-                        constexpr int K = (C::RING - 2) * C::BCH;
-                        __builtin_amdgcn_s_waitcnt((K & 15) | ((K >> 4) << 14) | (7 << 4) | (15 << 8));
+                        wait_vmcnt<(C::RING - 2) * C::BCH>();
                         issue_bias(t + C::RING - 1);  // into the slot block t - 1 has just left
                     } else {
                         load_bias_scalar(t, ring_lds + ((t - mb_first) & (C::RING - 1)) * C::BT_BYTES);
                     }
                 }
             }
-            const T* a_tile = s_wave ? q_lds : do_lds;
+            const T* a_tile = IS_S ? q_lds : do_lds;
 #pragma unroll
             for (int sb = 0; sb < NSUB; sb++) {
 #pragma unroll
@@ -608,7 +611,7 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
                 }
             }
         }
-        if (s_wave) {
+        if constexpr (IS_S) {
             if (live) {
                 // ---- P (flash_attention.py:281-294); register i of sub-block sb is row
                 // m0 + 32 sb + 8 (i/4) + 4 g + i%4, the lane is key my_n.  Blocks that touch a ragged
@@ -678,14 +681,16 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
                         acc[db] = mfma32(a, opT[sb][kk], acc[db]);
                     }
         }
-        __syncthreads();  // P(t) is visible to the dP-waves; nobody reads block t - 1's tiles any more
+        lds_barrier();  // P(t) is visible to the dP-waves; nobody reads block t - 1's tiles any more
 
         // =============================== second half ===============================
-        if (t + 1 < n_mblocks) {
-            stage_block(buf ^ 1);                            // block t + 1 -> LDS
-            if (t + 2 < n_mblocks) fetch_block(t + 2);       // block t + 2 -> registers
+        if constexpr (!IS_S) {
+            if (t + 1 < n_mblocks) {
+                stage_block(buf ^ 1);                        // block t + 1 -> LDS
+                if (t + 2 < n_mblocks) fetch_block(t + 2);   // block t + 2 -> registers
+            }
         }
-        if (s_wave) {
+        if constexpr (IS_S) {
             if (live) {
                 // ---- dV^T += dO^T P ----
 #pragma unroll
@@ -741,7 +746,14 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
                 }
             }
         }
-        __syncthreads();  // dS(t) and the tiles of block t + 1 are visible
+        lds_barrier();  // dS(t) and the tiles of block t + 1 are visible
+    };
+    if (s_wave) {
+#pragma unroll 1
+        for (int t = mb_first; t <= n_mblocks; t++) step(t, std::true_type{});
+    } else {
+#pragma unroll 1
+        for (int t = mb_first; t <= n_mblocks; t++) step(t, std::false_type{});
     }
 
     // ---- dV (S-wave) or dK (dP-wave) of this wave's 32 keys (flash_attention.py:449-454) ----

@@ -62,6 +62,15 @@ __device__ __forceinline__ float pair_sum(float x) {
     return __builtin_bit_cast(float, (int)r[0]) + __builtin_bit_cast(float, (int)r[1]);
 }
 
+// Work-group barrier that orders LDS traffic only.  Unlike __syncthreads() it does not wait for
+// outstanding global loads, stores or direct-to-LDS copies, so prefetches issued before it stay in
+// flight across it (a consumer of such a copy waits on vmcnt itself).
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 // ---- LDS access ---------------------------------------------------------------------------
 __device__ __forceinline__ i32x4 lds_read16(const void* p) { return *reinterpret_cast<const i32x4*>(p); }
 __device__ __forceinline__ void lds_write16(void* p, i32x4 v) { *reinterpret_cast<i32x4*>(p) = v; }
@@ -125,6 +134,32 @@ template <int D> struct Swz {
 __device__ __forceinline__ void g2lds16(const void* src, void* lds_base) {
     __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)src,
                                      (void __attribute__((address_space(3)))*)lds_base, 16, 0, 0);
+}
+
+// The same copy, issued behind the compiler's back.  The compiler makes every later LDS read that
+// might alias a direct-to-LDS copy wait for ALL outstanding vector-memory operations, which
+// empties a queue of copies issued several steps ahead.  Here it sees neither the LDS write nor
+// the vmcnt increment: the consumer must wait with an explicit s_waitcnt vmcnt(n) (copies
+// complete in issue order) before it reads the destination, and a wave that uses this must not
+// mix it with loads whose completion the compiler counts.  M0 is saved and restored.
+__device__ __forceinline__ void g2lds16_untracked(const void* src, void* lds_base) {
+    const unsigned lds_addr = __builtin_amdgcn_readfirstlane(
+        (unsigned)(uintptr_t)(__attribute__((address_space(3))) void*)lds_base);
+    unsigned saved_m0;
+    asm volatile(
+        "s_mov_b32 %0, m0\n\t"
+        "s_mov_b32 m0, %2\n\t"
+        "s_nop 0\n\t"
+        "global_load_lds_dwordx4 %1, off\n\t"
+        "s_nop 0\n\t"
+        "s_mov_b32 m0, %0"
+        : "=&s"(saved_m0)
+        : "v"(src), "s"(lds_addr)
+        : "memory");
+}
+// s_waitcnt vmcnt(n) alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14, the other counters maxed)
+template <int N> __device__ __forceinline__ void wait_vmcnt() {
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
 }
 
 // Raw buffer view of `bytes` bytes at `base` (16-byte aligned): loads beyond the end return 0 and

@@ -22,6 +22,8 @@ int check_problem(const fa_problem& p) {
     if (p.dtype != FA_F16 && p.dtype != FA_BF16) return FA_ERR_DTYPE;
     if (p.bias_dtype < FA_BIAS_NONE || p.bias_dtype > FA_BIAS_F32) return FA_ERR_DTYPE;
     if (p.causal && p.M != p.N) return FA_ERR_SHAPE;
+    // row indices times four (the LSE and delta vectors) are formed in 32 bits
+    if (p.M >= (1 << 28) || p.N >= (1 << 28)) return FA_ERR_SHAPE;
     // a grid is one-dimensional: tiles * B * H must fit in 31 bits
     if ((int64_t)((p.M + 63) / 64 + (p.N + 63) / 64) * p.B * p.H >= (1ll << 31)) return FA_ERR_SHAPE;
     return FA_OK;

@@ -350,7 +350,7 @@ __global__ __launch_bounds__(256, (RowCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_dq_
 // ---------------------------------------------------------------------------------------------
 template <int D, int BIAS> struct BwdCfg {
     static constexpr int BN = 128, NT = 512;
-    static constexpr int NSUB = (D <= 64 && BIAS != 4) ? 2 : 1;  // 32-row sub-blocks of a query block
+    static constexpr int NSUB = (D <= 64 && BIAS == 0) ? 2 : 1;  // 32-row sub-blocks of a query block
     static constexpr int BMI = 32 * NSUB;
     static constexpr int DP = D < 32 ? 32 : D;
     static constexpr int DB = DP / 32;
@@ -362,16 +362,21 @@ template <int D, int BIAS> struct BwdCfg {
     static constexpr int EPC = ES > 0 ? 16 / ES : 8;       // bias elements per 16-byte chunk
     static constexpr int BCPR = 2 * ES;                    // 16-byte chunks per 32-key bias row
     static constexpr int BCH = (BMI * BCPR + 63) / 64;     // bias chunks per lane per block
+    // LDS buffers of Q (+LSE) and of dO (+delta).  With four Q buffers the dK product of a block is
+    // deferred by a step (so that it does not wait for the dS of the same step); D = 256 has room
+    // for three only and runs it in the step of its dS.
+    static constexpr int NQB = D > 128 ? 3 : 4, NDOB = 2;
+    static constexpr bool DEFER_DK = NQB == 4;
     static constexpr int Q_BYTES = BMI * D * 2;
     static constexpr int DS_BYTES = BMI * DSS * 2;
     static constexpr int P_BYTES = 4 * NSUB * 64 * 64;     // P hand-off: 16 floats per lane per sub-block
-    static constexpr int STAT_BYTES = 2 * BMI * 4;
     static constexpr int BT_BYTES = BMI * 32 * ES;         // wave-private bias tile
-    static constexpr int OFF_DO = 2 * Q_BYTES;
-    static constexpr int OFF_DS = 4 * Q_BYTES;
-    static constexpr int OFF_P = OFF_DS + 2 * DS_BYTES;
-    static constexpr int OFF_STAT = OFF_P + P_BYTES;
-    static constexpr int OFF_BIAS = OFF_STAT + 2 * STAT_BYTES;
+    static constexpr int OFF_DO = NQB * Q_BYTES;
+    static constexpr int OFF_DS = OFF_DO + NDOB * Q_BYTES;
+    static constexpr int OFF_P = OFF_DS + DS_BYTES;        // two hand-off buffers
+    static constexpr int OFF_LSE = OFF_P + 2 * P_BYTES;
+    static constexpr int OFF_DELTA = OFF_LSE + NQB * BMI * 4;
+    static constexpr int OFF_BIAS = OFF_DELTA + NDOB * BMI * 4;
     // The bias slices of an S-wave arrive through a ring of RING LDS slots filled by direct
     // global -> LDS copies issued RING - 1 query blocks ahead: the bias is a pure HBM stream, and
     // only a deep queue keeps enough bytes in flight to cover the memory latency.
@@ -385,11 +390,13 @@ template <int D, int BIAS> struct BwdCfg {
 // pair up on the four 32-key blocks of the tile (waves w and w + 4 run on the same SIMD):
 //   S-wave : S = Q K^T, P = 2^(S*scale + bias - LSE)  -> hands P to its partner through LDS,
 //            dV^T += dO^T P
-//   dP-wave: dP = dO V^T, dS = P (dP - delta) (+ dBias through an LDS tile), dK^T += Q^T dS
-// A step handles one query block t and is cut in two by barriers so that in each half one wave
-// of a SIMD issues matrix instructions while the other does the exponentials / products:
-//   first half : S-wave: S(t), P(t)            dP-wave: dP(t), dK(t-1)
-//   second half: S-wave: dV(t)                 dP-wave: dS(t), dBias(t)
+//   dP-wave: dP = dO V^T, dS = P (dP - delta) (+ dBias through an LDS tile), dK^T += Q^T dS,
+//            and the global -> LDS staging of the Q / dO blocks
+// The roles are skewed by one query block so that a step needs a single barrier and nothing a
+// wave does inside a step depends on what its partner does in the same step:
+//   step t : S-wave : P(t+1) from Q(t+1), then dV += dO(t)^T P(t)        (P(t) kept in registers)
+//            dP-wave: dS(t) from dO(t) and the P(t) handed over in step t-1, dK += Q(t-1)^T dS(t-1)
+// While one wave of a SIMD runs exponentials or products the other issues MFMAs.
 template <typename T, int D, int BIAS, bool CAUSAL, bool DBIAS>
 __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
     typedef BwdCfg<D, BIAS> C;
@@ -428,7 +435,7 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
     if (BIAS != 0) bp = reinterpret_cast<const E*>(p.bias) + (int64_t)b * p.sbias.b + (int64_t)h * p.sbias.h;
     if (DBIAS) dbp = reinterpret_cast<E*>(p.dbias) + (int64_t)b * p.sdbias.b + (int64_t)h * p.sdbias.h;
     unsigned char* ring_lds = smem + C::OFF_BIAS + kb * C::RING * C::BT_BYTES;
-    float* p_lds = reinterpret_cast<float*>(smem + C::OFF_P) + kb * NSUB * 64 * 16;
+    float* p_lds = reinterpret_cast<float*>(smem + C::OFF_P) + kb * NSUB * 64 * 16;  // + buffer * P_BYTES / 4
 
     // ---- this wave's 32 keys as B operand (column my_n, k = d): K for an S-wave, V for a dP-wave
     T8 opreg[C::KSTEPS];
@@ -472,12 +479,16 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
         }
     }
 
-    // ---- global -> register staging, one query block ahead --------------------------------
-    // Q / dO rows through buffer views of this (b, h) slice: rows past M read as zero.
-    const __amdgpu_buffer_rsrc_t q_rsrc = make_buffer(qp, ((int64_t)(M - 1) * p.sq.s + D) * 2);
-    const __amdgpu_buffer_rsrc_t do_rsrc = make_buffer(dop, ((int64_t)(M - 1) * p.sdo.s + D) * 2);
-    // Only the dP-waves fetch tiles (and the LSE / delta rows): the S-waves keep their
-    // vector-memory queue for the deep bias prefetch, whose completion is counted in order.
+    // ---- global -> register -> LDS staging of Q (+LSE) and dO (+delta) blocks -------------
+    // Done by the dP-waves only: the S-waves keep their vector-memory queue for the deep bias
+    // prefetch, whose completion is counted in order.  Rows past M read as zero (buffer views).
+    // A buffer view per block: it starts at the block's first row and ends with the tensor, so
+    // that offsets inside it stay small whatever M is and a block past the end is an empty view.
+    auto block_view = [&](const T* base, int64_t row_stride, int mb) {
+        const int64_t rows_left = (int64_t)M - (int64_t)mb * BMI;
+        const int64_t bytes = rows_left > 0 ? ((rows_left - 1) * row_stride + D) * 2 : 0;
+        return make_buffer(base + (int64_t)mb * BMI * row_stride, bytes);
+    };
     const int ftid = tid - 256;  // thread index among the dP-waves
     int q_off[C::QCH], do_off[C::QCH];
 #pragma unroll
@@ -486,37 +497,47 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
         q_off[it] = (c / CPR) * (int)p.sq.s * 2 + (c % CPR) * 16;
         do_off[it] = (c / CPR) * (int)p.sdo.s * 2 + (c % CPR) * 16;
     }
+    const __amdgpu_buffer_rsrc_t lse_rsrc = make_buffer(lsep, (int64_t)M * 4);
+    const __amdgpu_buffer_rsrc_t delta_rsrc = make_buffer(deltap, (int64_t)M * 4);
     i32x4 qreg[C::QCH], doreg[C::QCH];
-    float stat_r = 0.f;
-    auto fetch_block = [&](int mb) {  // issue the loads of query block mb (dP-waves)
-        if (s_wave) return;
+    float lse_r = 0.f, delta_r = 0.f;
+    // Fetches and stores are unconditional: a block index past the end reads zeros (every offset is
+    // outside its buffer view) and lands in an LDS buffer that no one reads any more.  Straight-line
+    // code lets the loads of the next blocks stay in flight across the stores of this one.
+    auto fetch_q = [&](int mb) {
         const int m0 = mb * BMI;
+        const __amdgpu_buffer_rsrc_t q_rsrc = block_view(qp, p.sq.s, mb);
 #pragma unroll
-        for (int it = 0; it < C::QCH; it++) {
-            if (it * 256 + (ftid & ~63) < BMI * CPR) {  // wave-uniform
-                qreg[it] = buf_load16(q_rsrc, q_off[it], m0 * (int)p.sq.s * 2);
-                doreg[it] = buf_load16(do_rsrc, do_off[it], m0 * (int)p.sdo.s * 2);
-            }
-        }
-        if (ftid < 2 * BMI) {
-            const int m = m0 + (ftid & (BMI - 1));
-            const float* src = ftid < BMI ? lsep : deltap;
-            stat_r = m < M ? src[m] : 0.f;
-        }
+        for (int it = 0; it < C::QCH; it++)
+            if (it * 256 + (ftid & ~63) < BMI * CPR) qreg[it] = buf_load16(q_rsrc, q_off[it], 0);
+        if (ftid < BMI) lse_r = buf_load_f32(lse_rsrc, (m0 + ftid) * 4, 0);
     };
-    auto stage_block = [&](int buf) {  // registers -> LDS tiles of buffer `buf` (dP-waves)
-        if (s_wave) return;
-        T* q_lds = reinterpret_cast<T*>(smem + buf * C::Q_BYTES);
-        T* do_lds = reinterpret_cast<T*>(smem + C::OFF_DO + buf * C::Q_BYTES);
+    auto stage_q = [&](int mb) {
+        T* dst = reinterpret_cast<T*>(smem + (mb % C::NQB) * C::Q_BYTES);
 #pragma unroll
         for (int it = 0; it < C::QCH; it++) {
             const int c = it * 256 + ftid;
-            if (c < BMI * CPR) {
-                lds_write16(q_lds + SW::off(c / CPR, (c % CPR) * 8), qreg[it]);
-                lds_write16(do_lds + SW::off(c / CPR, (c % CPR) * 8), doreg[it]);
-            }
+            if (c < BMI * CPR) lds_write16(dst + SW::off(c / CPR, (c % CPR) * 8), qreg[it]);
         }
-        if (ftid < 2 * BMI) reinterpret_cast<float*>(smem + C::OFF_STAT + buf * C::STAT_BYTES)[ftid] = stat_r;
+        if (ftid < BMI) reinterpret_cast<float*>(smem + C::OFF_LSE)[(mb % C::NQB) * BMI + ftid] = lse_r;
+    };
+    auto fetch_do = [&](int mb) {
+        const int m0 = mb * BMI;
+        const __amdgpu_buffer_rsrc_t do_rsrc = block_view(dop, p.sdo.s, mb);
+#pragma unroll
+        for (int it = 0; it < C::QCH; it++)
+            if (it * 256 + (ftid & ~63) < BMI * CPR) doreg[it] = buf_load16(do_rsrc, do_off[it], 0);
+        if (ftid >= 256 - BMI) delta_r = buf_load_f32(delta_rsrc, (m0 + ftid - (256 - BMI)) * 4, 0);
+    };
+    auto stage_do = [&](int mb) {
+        T* dst = reinterpret_cast<T*>(smem + C::OFF_DO + (mb & (C::NDOB - 1)) * C::Q_BYTES);
+#pragma unroll
+        for (int it = 0; it < C::QCH; it++) {
+            const int c = it * 256 + ftid;
+            if (c < BMI * CPR) lds_write16(dst + SW::off(c / CPR, (c % CPR) * 8), doreg[it]);
+        }
+        if (ftid >= 256 - BMI)
+            reinterpret_cast<float*>(smem + C::OFF_DELTA)[(mb & (C::NDOB - 1)) * BMI + ftid - (256 - BMI)] = delta_r;
     };
 
     // bias slice (BMI rows x 32 keys) of query block mb -> ring slot, straight from HBM to LDS.
@@ -554,65 +575,77 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
         }
     };
 
+    // ---- prologue: Q(first) staged, Q(first+1) and dO(first) on their way ----
     if (mb_first < n_mblocks) {
-        fetch_block(mb_first);
-        stage_block(mb_first & 1);
-        if (mb_first + 1 < n_mblocks) fetch_block(mb_first + 1);
-        if (BIAS != 0 && s_wave && bias_vec) {
+        if (!s_wave) {
+            fetch_q(mb_first);
+            stage_q(mb_first);
+            fetch_q(mb_first + 1);
+            fetch_do(mb_first);
+        } else if (BIAS != 0 && bias_vec) {
 #pragma unroll 1
             for (int mb = mb_first; mb < mb_first + C::RING - 1; mb++) issue_bias(mb);
         }
     }
     __syncthreads();
 
-    T8 opT[NSUB][2];  // P^T (S-wave) or dS^T (dP-wave) of the current block, packed as B operands
+    T8 op_cur[NSUB][2];  // P^T (S-wave) or dS^T (dP-wave) of the block whose accumulation is still due
+#pragma unroll
+    for (int sb = 0; sb < NSUB; sb++)
+#pragma unroll
+        for (int kk = 0; kk < 2; kk++) op_cur[sb][kk] = as_vec<T8>(i32x4{0, 0, 0, 0});
 
-    // One step of the pipeline for one role.  The two roles run separate instances of the loop
-    // (same number of barriers each), so that the compiler's memory-wait bookkeeping of one role
-    // (tile loads counted by the compiler) never leaks into the other (bias copies counted by hand).
-    auto step = [&](int t, auto role_tag) {
-        constexpr bool IS_S = decltype(role_tag)::value;
-        const int buf = t & 1;
-        const bool live = t < n_mblocks;  // block t exists (the last step only drains block t - 1)
-        const bool prev = t > mb_first;   // block t - 1 exists
-        const int m0 = t * BMI;
-        const T* q_lds = reinterpret_cast<const T*>(smem + buf * C::Q_BYTES);
-        const T* do_lds = reinterpret_cast<const T*>(smem + C::OFF_DO + buf * C::Q_BYTES);
-        const T* q_prev = reinterpret_cast<const T*>(smem + (buf ^ 1) * C::Q_BYTES);
-        T* ds_cur = reinterpret_cast<T*>(smem + C::OFF_DS + buf * C::DS_BYTES);
-        const float* stat_lds = reinterpret_cast<const float*>(smem + C::OFF_STAT + buf * C::STAT_BYTES);
-        const bool need_mask = (m0 + BMI > M) || (n0 + BN > N) || (CAUSAL && m0 < n0 + BN - 1);
-        const unsigned char* bt_lds = ring_lds + ((t - mb_first) & (C::RING - 1)) * C::BT_BYTES;
-
-        // =============================== first half ===============================
-        f32x16 sacc[NSUB];  // S (S-wave) or dP (dP-wave)
-        if (live) {
-            if constexpr (BIAS != 0 && IS_S) {
-                {
-                    if (bias_vec) {
-                        // the copies of block t were issued RING - 1 steps ago and at most the
-                        // (RING - 2) * BCH copies issued since may still be in flight
-                        wait_vmcnt<(C::RING - 2) * C::BCH>();
-                        issue_bias(t + C::RING - 1);  // into the slot block t - 1 has just left
-                    } else {
-                        load_bias_scalar(t, ring_lds + ((t - mb_first) & (C::RING - 1)) * C::BT_BYTES);
-                    }
-                }
-            }
-            const T* a_tile = IS_S ? q_lds : do_lds;
+    // sacc = rows(tile) x opreg: S = Q K^T (S-wave) or dP = dO V^T (dP-wave)
+    auto gemm_rows = [&](const T* tile, f32x16 (&sacc)[NSUB]) {
 #pragma unroll
-            for (int sb = 0; sb < NSUB; sb++) {
+        for (int sb = 0; sb < NSUB; sb++) {
 #pragma unroll
-                for (int i = 0; i < 16; i++) sacc[sb][i] = 0.f;
+            for (int i = 0; i < 16; i++) sacc[sb][i] = 0.f;
 #pragma unroll
-                for (int ks = 0; ks < C::KSTEPS; ks++) {
-                    T8 a = as_vec<T8>(lds_read16(a_tile + SW::off(sb * 32 + r, ks * 16 + 8 * g)));
-                    sacc[sb] = mfma32(a, opreg[ks], sacc[sb]);
-                }
+            for (int ks = 0; ks < C::KSTEPS; ks++) {
+                T8 a = as_vec<T8>(lds_read16(tile + SW::off(sb * 32 + r, ks * 16 + 8 * g)));
+                sacc[sb] = mfma32(a, opreg[ks], sacc[sb]);
             }
         }
-        if constexpr (IS_S) {
-            if (live) {
+    };
+    // acc^T += tile^T op: dV^T += dO^T P (S-wave) or dK^T += Q^T dS (dP-wave); the A operands are
+    // columns of the tile gathered with ds_read_b64_tr_b16
+    auto gemm_cols = [&](const T* tile, const T8 (&op)[NSUB][2]) {
+#pragma unroll
+        for (int sb = 0; sb < NSUB; sb++)
+#pragma unroll
+            for (int kk = 0; kk < 2; kk++)
+#pragma unroll
+                for (int db = 0; db < C::DB; db++) {
+                    T8 a = SW::template col8<T8>(tile, lane, sb * 32 + kk * 16, db * 32);
+                    acc[db] = mfma32(a, op[sb][kk], acc[db]);
+                }
+    };
+
+    if (s_wave) {
+        // ================================ S-wave ================================
+#pragma unroll 1
+        for (int t = mb_first - 1; t <= n_mblocks; t++) {
+            const int nb = t + 1;  // the block whose P is produced in this step
+            T8 op_next[NSUB][2];
+            if (nb < n_mblocks) {
+                const int m0 = nb * BMI;
+                const unsigned char* bt_lds = ring_lds + ((nb - mb_first) & (C::RING - 1)) * C::BT_BYTES;
+                if constexpr (BIAS != 0) {
+                    if (bias_vec) {
+                        // the copies of block nb were issued RING - 1 steps ago and at most the
+                        // (RING - 2) * BCH copies issued since may still be in flight
+                        wait_vmcnt<(C::RING - 2) * C::BCH>();
+                        issue_bias(nb + C::RING - 1);  // into the slot the previous block has left
+                    } else {
+                        load_bias_scalar(nb, ring_lds + ((nb - mb_first) & (C::RING - 1)) * C::BT_BYTES);
+                    }
+                }
+                const bool need_mask = (m0 + BMI > M) || (n0 + BN > N) || (CAUSAL && m0 < n0 + BN - 1);
+                f32x16 sacc[NSUB];
+                gemm_rows(reinterpret_cast<const T*>(smem + (nb % C::NQB) * C::Q_BYTES), sacc);
+                const float* lse_lds = reinterpret_cast<const float*>(smem + C::OFF_LSE) + (nb % C::NQB) * BMI;
+                float* p_out = p_lds + (nb & 1) * (C::P_BYTES / 4);
                 // ---- P (flash_attention.py:281-294); register i of sub-block sb is row
                 // m0 + 32 sb + 8 (i/4) + 4 g + i%4, the lane is key my_n.  Blocks that touch a ragged
                 // edge or the causal diagonal follow the reference's additive -1e6 arithmetic term by
@@ -624,7 +657,7 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
 #pragma unroll
                         for (int q4 = 0; q4 < 4; q4++) {
                             const int ml0 = sb * 32 + 8 * q4 + 4 * g;  // first of 4 consecutive rows
-                            const f32x4 lse4 = *reinterpret_cast<const f32x4*>(stat_lds + ml0);
+                            const f32x4 lse4 = *reinterpret_cast<const f32x4*>(lse_lds + ml0);
                             float bv[4] = {0.f, 0.f, 0.f, 0.f};  // bias in log2 units / mask term
                             if constexpr (BIAS == 1) {
 #pragma unroll
@@ -659,101 +692,87 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
                                     pv = fast_exp2(__builtin_fmaf(sacc[sb][i], qk_scale, bv[e] - lse4[e]));
                                 }
                                 p4[e] = pv;
-                                opT[sb][i >> 3][i & 7] = (T)pv;
+                                op_next[sb][i >> 3][i & 7] = (T)pv;
                             }
                             // hand P to the dP-wave of the same keys: same lane, same register order
-                            *reinterpret_cast<f32x4*>(p_lds + ((sb * 4 + q4) * 64 + lane) * 4) = p4;
+                            *reinterpret_cast<f32x4*>(p_out + ((sb * 4 + q4) * 64 + lane) * 4) = p4;
                         }
                     }
                 };
                 if (need_mask) p_step(std::true_type{});
                 else p_step(std::false_type{});
             }
-        } else if (prev) {
-            // ---- dK^T += Q^T dS of the previous block ----
+            if (t >= mb_first && t < n_mblocks)  // dV^T += dO(t)^T P(t)
+                gemm_cols(reinterpret_cast<const T*>(smem + C::OFF_DO + (t & (C::NDOB - 1)) * C::Q_BYTES), op_cur);
 #pragma unroll
             for (int sb = 0; sb < NSUB; sb++)
 #pragma unroll
-                for (int kk = 0; kk < 2; kk++)
-#pragma unroll
-                    for (int db = 0; db < C::DB; db++) {
-                        T8 a = SW::template col8<T8>(q_prev, lane, sb * 32 + kk * 16, db * 32);
-                        acc[db] = mfma32(a, opT[sb][kk], acc[db]);
-                    }
+                for (int kk = 0; kk < 2; kk++) op_cur[sb][kk] = op_next[sb][kk];
+            lds_barrier();
         }
-        lds_barrier();  // P(t) is visible to the dP-waves; nobody reads block t - 1's tiles any more
-
-        // =============================== second half ===============================
-        if constexpr (!IS_S) {
-            if (t + 1 < n_mblocks) {
-                stage_block(buf ^ 1);                        // block t + 1 -> LDS
-                if (t + 2 < n_mblocks) fetch_block(t + 2);   // block t + 2 -> registers
-            }
-        }
-        if constexpr (IS_S) {
-            if (live) {
-                // ---- dV^T += dO^T P ----
-#pragma unroll
-                for (int sb = 0; sb < NSUB; sb++)
-#pragma unroll
-                    for (int kk = 0; kk < 2; kk++)
-#pragma unroll
-                        for (int db = 0; db < C::DB; db++) {
-                            T8 a = SW::template col8<T8>(do_lds, lane, sb * 32 + kk * 16, db * 32);
-                            acc[db] = mfma32(a, opT[sb][kk], acc[db]);
-                        }
-            }
-        } else if (live) {
-            // ---- dS = P (dP - delta) (flash_attention.py:303-308) ----
-            const float* delta_lds = stat_lds + BMI;
-#pragma unroll
-            for (int sb = 0; sb < NSUB; sb++) {
-#pragma unroll
-                for (int q4 = 0; q4 < 4; q4++) {
-                    const int ml0 = sb * 32 + 8 * q4 + 4 * g;
-                    const f32x4 del4 = *reinterpret_cast<const f32x4*>(delta_lds + ml0);
-                    const f32x4 p4 = *reinterpret_cast<const f32x4*>(p_lds + ((sb * 4 + q4) * 64 + lane) * 4);
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        const int i = q4 * 4 + e;
-                        const float dsv = p4[e] * (sacc[sb][i] - del4[e]);
-                        opT[sb][i >> 3][i & 7] = (T)dsv;
-                        ds_cur[(ml0 + e) * DSS + kb * 32 + r] = (T)dsv;
-                        if constexpr (DBIAS && !DB_VIA_LDS) {
-                            const int m = m0 + ml0 + e;
-                            if (m < M && my_n < N) dbp[(int64_t)m * p.sdbias.m + (int64_t)my_n * p.sdbias.n] = (E)dsv;
-                        }
-                    }
-                }
-            }
-            // ---- dBias rows of this wave's 32 keys, 16 bytes per lane, out of the dS tile ----
-            if constexpr (DB_VIA_LDS) {
-#pragma unroll
-                for (int it = 0; it < (BMI * 4) / 64; it++) {
-                    const int c = it * 64 + lane;
-                    const int row = c >> 2, ch = c & 3;
-                    const int m = m0 + row, nn = nw + ch * 8;
-                    if (m < M && nn < N) {
-                        const T* src = ds_cur + row * DSS + kb * 32 + ch * 8;
-                        E* dst = dbp + (int64_t)m * p.sdbias.m + (int64_t)nn * p.sdbias.n;
-                        if (dbias_vec && nn + 8 <= N) {
-                            gst16(dst, lds_read16(src));
-                        } else {
-                            for (int e = 0; e < 8; e++)
-                                if (nn + e < N) dst[(int64_t)e * p.sdbias.n] = __builtin_bit_cast(E, src[e]);
-                        }
-                    }
-                }
-            }
-        }
-        lds_barrier();  // dS(t) and the tiles of block t + 1 are visible
-    };
-    if (s_wave) {
-#pragma unroll 1
-        for (int t = mb_first; t <= n_mblocks; t++) step(t, std::true_type{});
     } else {
+        // ================================ dP-wave ================================
+        T* ds_lds = reinterpret_cast<T*>(smem + C::OFF_DS);
 #pragma unroll 1
-        for (int t = mb_first; t <= n_mblocks; t++) step(t, std::false_type{});
+        for (int t = mb_first - 1; t <= n_mblocks; t++) {
+            // blocks on their way: Q(t+2), dO(t+1) registers -> LDS; Q(t+3), dO(t+2) -> registers
+            stage_q(t + 2);
+            stage_do(t + 1);
+            fetch_q(t + 3);
+            fetch_do(t + 2);
+            if (C::DEFER_DK && t - 1 >= mb_first)  // dK^T += Q(t-1)^T dS(t-1)
+                gemm_cols(reinterpret_cast<const T*>(smem + ((t - 1) % C::NQB) * C::Q_BYTES), op_cur);
+            if (t >= mb_first && t < n_mblocks) {
+                const int m0 = t * BMI;
+                f32x16 sacc[NSUB];
+                gemm_rows(reinterpret_cast<const T*>(smem + C::OFF_DO + (t & (C::NDOB - 1)) * C::Q_BYTES), sacc);
+                // ---- dS = P (dP - delta) (flash_attention.py:303-308) ----
+                const float* delta_lds = reinterpret_cast<const float*>(smem + C::OFF_DELTA) + (t & (C::NDOB - 1)) * BMI;
+                const float* p_in = p_lds + (t & 1) * (C::P_BYTES / 4);
+#pragma unroll
+                for (int sb = 0; sb < NSUB; sb++) {
+#pragma unroll
+                    for (int q4 = 0; q4 < 4; q4++) {
+                        const int ml0 = sb * 32 + 8 * q4 + 4 * g;
+                        const f32x4 del4 = *reinterpret_cast<const f32x4*>(delta_lds + ml0);
+                        const f32x4 p4 = *reinterpret_cast<const f32x4*>(p_in + ((sb * 4 + q4) * 64 + lane) * 4);
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            const int i = q4 * 4 + e;
+                            const float dsv = p4[e] * (sacc[sb][i] - del4[e]);
+                            op_cur[sb][i >> 3][i & 7] = (T)dsv;
+                            if constexpr (DB_VIA_LDS) ds_lds[(ml0 + e) * DSS + kb * 32 + r] = (T)dsv;
+                            if constexpr (DBIAS && !DB_VIA_LDS) {
+                                const int m = m0 + ml0 + e;
+                                if (m < M && my_n < N) dbp[(int64_t)m * p.sdbias.m + (int64_t)my_n * p.sdbias.n] = (E)dsv;
+                            }
+                        }
+                    }
+                }
+                // ---- dBias rows of this wave's 32 keys, 16 bytes per lane, out of the dS tile ----
+                if constexpr (DB_VIA_LDS) {
+#pragma unroll
+                    for (int it = 0; it < (BMI * 4) / 64; it++) {
+                        const int c = it * 64 + lane;
+                        const int row = c >> 2, ch = c & 3;
+                        const int m = m0 + row, nn = nw + ch * 8;
+                        if (m < M && nn < N) {
+                            const T* src = ds_lds + row * DSS + kb * 32 + ch * 8;
+                            E* dst = dbp + (int64_t)m * p.sdbias.m + (int64_t)nn * p.sdbias.n;
+                            if (dbias_vec && nn + 8 <= N) {
+                                gst16(dst, lds_read16(src));
+                            } else {
+                                for (int e = 0; e < 8; e++)
+                                    if (nn + e < N) dst[(int64_t)e * p.sdbias.n] = __builtin_bit_cast(E, src[e]);
+                            }
+                        }
+                    }
+                }
+                if (!C::DEFER_DK)  // dK^T += Q(t)^T dS(t)
+                    gemm_cols(reinterpret_cast<const T*>(smem + (t % C::NQB) * C::Q_BYTES), op_cur);
+            }
+            lds_barrier();
+        }
     }
 
     // ---- dV (S-wave) or dK (dP-wave) of this wave's 32 keys (flash_attention.py:449-454) ----

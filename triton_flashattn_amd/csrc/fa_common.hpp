@@ -172,6 +172,9 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_buffer(const void* base, 
     const unsigned n = bytes < 0 ? 0u : (unsigned)(bytes > cap ? cap : bytes);
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)n, 0x00020000);
 }
+__device__ __forceinline__ float buf_load_f32(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
+}
 __device__ __forceinline__ i32x4 buf_load16(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
     return __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
 }

@@ -713,6 +713,24 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
     } else {
         // ================================ dP-wave ================================
         T* ds_lds = reinterpret_cast<T*>(smem + C::OFF_DS);
+        // dBias rows that are whole aligned 16-byte chunks leave through unconditional buffer
+        // stores (chunks outside the tensor get an offset outside the view): a loop without
+        // branches around its stores lets the loads of the next blocks stay in flight across them.
+        const bool db_fast = DB_VIA_LDS && dbias_vec && (N % 8 == 0);
+        __amdgpu_buffer_rsrc_t db_rsrc = make_buffer(nullptr, 0);
+        int db_off[(BMI * 4) / 64];
+        const int db_row_bytes = DB_VIA_LDS ? (int)p.sdbias.m * 2 : 0;
+        if (db_fast) {
+            db_rsrc = make_buffer(dbp, ((int64_t)(M - 1) * p.sdbias.m + N) * 2);
+#pragma unroll
+            for (int it = 0; it < (BMI * 4) / 64; it++) {
+                const int c = it * 64 + lane;
+                const int nn = nw + (c & 3) * 8;
+                db_off[it] = nn < N ? (c >> 2) * db_row_bytes + nn * 2 : (int)0x80000000;
+            }
+        }
+        auto dp_loop = [&](auto fast_tag) {
+        constexpr bool DB_FAST = decltype(fast_tag)::value;
 #pragma unroll 1
         for (int t = mb_first - 1; t <= n_mblocks; t++) {
             // blocks on their way: Q(t+2), dO(t+1) registers -> LDS; Q(t+3), dO(t+2) -> registers
@@ -756,7 +774,13 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
                         const int c = it * 64 + lane;
                         const int row = c >> 2, ch = c & 3;
                         const int m = m0 + row, nn = nw + ch * 8;
-                        if (m < M && nn < N) {
+                        if constexpr (DB_FAST) {
+                            const T* src = ds_lds + row * DSS + kb * 32 + ch * 8;
+                            // rows past M: m0 * row bytes alone is past the view only if the view is
+                            // tight, so the row test is explicit
+                            const int off = m < M ? db_off[it] + m0 * db_row_bytes : (int)0x80000000;
+                            buf_store16(db_rsrc, lds_read16(src), off);
+                        } else if (m < M && nn < N) {
                             const T* src = ds_lds + row * DSS + kb * 32 + ch * 8;
                             E* dst = dbp + (int64_t)m * p.sdbias.m + (int64_t)nn * p.sdbias.n;
                             if (dbias_vec && nn + 8 <= N) {
@@ -772,6 +796,13 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
                     gemm_cols(reinterpret_cast<const T*>(smem + (t % C::NQB) * C::Q_BYTES), op_cur);
             }
             lds_barrier();
+        }
+        };
+        if constexpr (DB_VIA_LDS) {
+            if (db_fast) dp_loop(std::true_type{});
+            else dp_loop(std::false_type{});
+        } else {
+            dp_loop(std::false_type{});
         }
     }
 

@@ -172,6 +172,10 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_buffer(const void* base, 
     const unsigned n = bytes < 0 ? 0u : (unsigned)(bytes > cap ? cap : bytes);
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)n, 0x00020000);
 }
+// 16-byte store through a buffer view; an offset outside the view drops the store
+__device__ __forceinline__ void buf_store16(__amdgpu_buffer_rsrc_t r, i32x4 v, int voff) {
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(__attribute__((__vector_size__(4 * sizeof(unsigned int)))) unsigned int, v), r, voff, 0, 0);
+}
 __device__ __forceinline__ float buf_load_f32(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
     return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
 }

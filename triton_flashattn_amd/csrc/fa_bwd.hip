@@ -356,32 +356,37 @@ template <int D, int BIAS> struct BwdCfg {
     static constexpr int DB = DP / 32;
     static constexpr int KSTEPS = D / 16;
     static constexpr int CPR = D / 8;
-    static constexpr int QCH = (BMI * CPR + 255) / 256;    // 16-byte chunks per dP-wave thread per Q (or dO) block
     static constexpr int DSS = BN + 8;                     // dS tile row stride (elements)
     static constexpr int ES = BIAS == 0 ? 0 : (BIAS == 1 ? 1 : (BIAS == 4 ? 4 : 2));
     static constexpr int EPC = ES > 0 ? 16 / ES : 8;       // bias elements per 16-byte chunk
     static constexpr int BCPR = 2 * ES;                    // 16-byte chunks per 32-key bias row
-    static constexpr int BCH = (BMI * BCPR + 63) / 64;     // bias chunks per lane per block
-    // LDS buffers of Q (+LSE) and of dO (+delta).  With four Q buffers the dK product of a block is
-    // deferred by a step (so that it does not wait for the dS of the same step); D = 256 has room
-    // for three only and runs it in the step of its dS.
-    static constexpr int NQB = D > 128 ? 3 : 4, NDOB = 2;
-    static constexpr bool DEFER_DK = NQB == 4;
+    static constexpr int BCH = (BMI * BCPR + 63) / 64;     // bias copies per S-wave per block
     static constexpr int Q_BYTES = BMI * D * 2;
-    static constexpr int DS_BYTES = BMI * DSS * 2;
+    static constexpr int NQD = Q_BYTES / 1024;             // 1 KB copies per Q (or dO) block
+    static constexpr int QD = NQD >= 4 ? NQD / 4 : 1;      // of which each S-wave issues this many
+    // Q, dO, LSE, delta and the bias slices reach LDS through direct global -> LDS copies that the
+    // S-waves issue LA blocks ahead of their use; a copy has LA - 1 whole steps and the rest of
+    // its own to land before the barrier that publishes it.
+    static constexpr int DS_BYTES = (BIAS == 2 || BIAS == 3) ? BMI * DSS * 2 : 0;  // dS tile (dBias)
     static constexpr int P_BYTES = 4 * NSUB * 64 * 64;     // P hand-off: 16 floats per lane per sub-block
-    static constexpr int BT_BYTES = BMI * 32 * ES;         // wave-private bias tile
+    static constexpr int BT_BYTES = BMI * 32 * ES;         // bias slice of one S-wave
+    // LDS bytes with copies la blocks ahead: la + 1 dO buffers and bias slots, la + 2 Q buffers and
+    // one more if the dK product of a block is deferred by a step (so that it does not wait for
+    // the dS of the same step)
+    static constexpr int lds_total(int la, int defer) {
+        return (2 * la + 3 + defer) * (Q_BYTES + BMI * 4) + DS_BYTES + 2 * P_BYTES + 4 * (la + 1) * BT_BYTES;
+    }
+    static constexpr int LA = D > 128 ? 1 : (lds_total(3, 1) <= 163840 ? 3 : 2);
+    static constexpr bool DEFER_DK = D <= 128 && lds_total(LA, 1) <= 163840;
+    static constexpr int NDOB = LA + 1;                    // dO (+delta) buffers
+    static constexpr int RING = LA + 1;                    // bias slots per S-wave
+    static constexpr int NQB = LA + 2 + (DEFER_DK ? 1 : 0);  // Q (+LSE) buffers
     static constexpr int OFF_DO = NQB * Q_BYTES;
     static constexpr int OFF_DS = OFF_DO + NDOB * Q_BYTES;
     static constexpr int OFF_P = OFF_DS + DS_BYTES;        // two hand-off buffers
     static constexpr int OFF_LSE = OFF_P + 2 * P_BYTES;
     static constexpr int OFF_DELTA = OFF_LSE + NQB * BMI * 4;
     static constexpr int OFF_BIAS = OFF_DELTA + NDOB * BMI * 4;
-    // The bias slices of an S-wave arrive through a ring of RING LDS slots filled by direct
-    // global -> LDS copies issued RING - 1 query blocks ahead: the bias is a pure HBM stream, and
-    // only a deep queue keeps enough bytes in flight to cover the memory latency.
-    static constexpr int RING_FIT = BT_BYTES > 0 ? (163840 - OFF_BIAS) / (4 * BT_BYTES) : 0;
-    static constexpr int RING = RING_FIT >= 8 ? 8 : (RING_FIT >= 4 ? 4 : 2);
     static constexpr int LOOP_BYTES = OFF_BIAS + 4 * RING * BT_BYTES;
     static constexpr int LDS_BYTES = LOOP_BYTES;
 };
@@ -390,8 +395,8 @@ template <int D, int BIAS> struct BwdCfg {
 // pair up on the four 32-key blocks of the tile (waves w and w + 4 run on the same SIMD):
 //   S-wave : S = Q K^T, P = 2^(S*scale + bias - LSE)  -> hands P to its partner through LDS,
 //            dV^T += dO^T P
-//   dP-wave: dP = dO V^T, dS = P (dP - delta) (+ dBias through an LDS tile), dK^T += Q^T dS,
-//            and the global -> LDS staging of the Q / dO blocks
+//            and the global -> LDS copies of the Q / dO / LSE / delta / bias blocks
+//   dP-wave: dP = dO V^T, dS = P (dP - delta) (+ dBias through an LDS tile), dK^T += Q^T dS
 // The roles are skewed by one query block so that a step needs a single barrier and nothing a
 // wave does inside a step depends on what its partner does in the same step:
 //   step t : S-wave : P(t+1) from Q(t+1), then dV += dO(t)^T P(t)        (P(t) kept in registers)
@@ -479,81 +484,59 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
         }
     }
 
-    // ---- global -> register -> LDS staging of Q (+LSE) and dO (+delta) blocks -------------
-    // Done by the dP-waves only: the S-waves keep their vector-memory queue for the deep bias
-    // prefetch, whose completion is counted in order.  Rows past M read as zero (buffer views).
-    // A buffer view per block: it starts at the block's first row and ends with the tensor, so
-    // that offsets inside it stay small whatever M is and a block past the end is an empty view.
-    auto block_view = [&](const T* base, int64_t row_stride, int mb) {
-        const int64_t rows_left = (int64_t)M - (int64_t)mb * BMI;
-        const int64_t bytes = rows_left > 0 ? ((rows_left - 1) * row_stride + D) * 2 : 0;
-        return make_buffer(base + (int64_t)mb * BMI * row_stride, bytes);
-    };
-    const int ftid = tid - 256;  // thread index among the dP-waves
-    int q_off[C::QCH], do_off[C::QCH];
+    // ---- global -> LDS copies of Q (+LSE), dO (+delta) and bias blocks, issued by the S-waves ----
+    // A block is NQD copies of 1 KB; copy ci fills bytes [1024 ci, 1024 ci + 1024) of the swizzled
+    // tile, so lane l of it fetches the 16-byte chunk that lives at tile position 64 ci + l.  Each
+    // S-wave issues QD of them (more than once where a block has fewer than four), every step the
+    // same number: completion is counted (s_waitcnt vmcnt) and copies complete in issue order.
+    // Rows past M re-read the last row: their P and dS are exactly zero.
+    unsigned cq_off[C::QD], cdo_off[C::QD];
+    int c_idx[C::QD];
 #pragma unroll
-    for (int it = 0; it < C::QCH; it++) {
-        const int c = it * 256 + (ftid & 255);
-        q_off[it] = (c / CPR) * (int)p.sq.s * 2 + (c % CPR) * 16;
-        do_off[it] = (c / CPR) * (int)p.sdo.s * 2 + (c % CPR) * 16;
+    for (int i = 0; i < C::QD; i++) {
+        c_idx[i] = (kb * C::QD + i) % C::NQD;
+        const int c = c_idx[i] * 64 + lane;
+        const int row = c / CPR, src = (c % CPR) ^ SW::f(row);
+        cq_off[i] = (unsigned)(row * (int)p.sq.s * 2 + src * 16);
+        cdo_off[i] = (unsigned)(row * (int)p.sdo.s * 2 + src * 16);
     }
-    const __amdgpu_buffer_rsrc_t lse_rsrc = make_buffer(lsep, (int64_t)M * 4);
-    const __amdgpu_buffer_rsrc_t delta_rsrc = make_buffer(deltap, (int64_t)M * 4);
-    i32x4 qreg[C::QCH], doreg[C::QCH];
-    float lse_r = 0.f, delta_r = 0.f;
-    // Fetches and stores are unconditional: a block index past the end reads zeros (every offset is
-    // outside its buffer view) and lands in an LDS buffer that no one reads any more.  Straight-line
-    // code lets the loads of the next blocks stay in flight across the stores of this one.
-    auto fetch_q = [&](int mb) {
-        const int m0 = mb * BMI;
-        const __amdgpu_buffer_rsrc_t q_rsrc = block_view(qp, p.sq.s, mb);
+    auto issue_rows = [&](const T* base, int64_t row_stride, const unsigned (&off)[C::QD], int mb, unsigned char* dst) {
+        // a block past the end is the last row over and over: offsets never go negative
+        const int m0 = mb * BMI < M ? mb * BMI : M - 1;
+        const T* blk = base + (int64_t)m0 * row_stride;
+        const bool full = m0 + BMI <= M;
 #pragma unroll
-        for (int it = 0; it < C::QCH; it++)
-            if (it * 256 + (ftid & ~63) < BMI * CPR) qreg[it] = buf_load16(q_rsrc, q_off[it], 0);
-        if (ftid < BMI) lse_r = buf_load_f32(lse_rsrc, (m0 + ftid) * 4, 0);
-    };
-    auto stage_q = [&](int mb) {
-        T* dst = reinterpret_cast<T*>(smem + (mb % C::NQB) * C::Q_BYTES);
-#pragma unroll
-        for (int it = 0; it < C::QCH; it++) {
-            const int c = it * 256 + ftid;
-            if (c < BMI * CPR) lds_write16(dst + SW::off(c / CPR, (c % CPR) * 8), qreg[it]);
+        for (int i = 0; i < C::QD; i++) {
+            unsigned o = off[i];
+            if (!full) {
+                const int c = c_idx[i] * 64 + lane;
+                int row = c / CPR;
+                const int src = (c % CPR) ^ SW::f(row);
+                row = row < M - m0 ? row : M - 1 - m0;
+                o = (unsigned)(row * (int)row_stride * 2 + src * 16);
+            }
+            g2lds16_untracked(blk, o, dst + c_idx[i] * 1024);
         }
-        if (ftid < BMI) reinterpret_cast<float*>(smem + C::OFF_LSE)[(mb % C::NQB) * BMI + ftid] = lse_r;
     };
-    auto fetch_do = [&](int mb) {
-        const int m0 = mb * BMI;
-        const __amdgpu_buffer_rsrc_t do_rsrc = block_view(dop, p.sdo.s, mb);
-#pragma unroll
-        for (int it = 0; it < C::QCH; it++)
-            if (it * 256 + (ftid & ~63) < BMI * CPR) doreg[it] = buf_load16(do_rsrc, do_off[it], 0);
-        if (ftid >= 256 - BMI) delta_r = buf_load_f32(delta_rsrc, (m0 + ftid - (256 - BMI)) * 4, 0);
-    };
-    auto stage_do = [&](int mb) {
-        T* dst = reinterpret_cast<T*>(smem + C::OFF_DO + (mb & (C::NDOB - 1)) * C::Q_BYTES);
-#pragma unroll
-        for (int it = 0; it < C::QCH; it++) {
-            const int c = it * 256 + ftid;
-            if (c < BMI * CPR) lds_write16(dst + SW::off(c / CPR, (c % CPR) * 8), doreg[it]);
+    // one float per row: the even S-waves copy LSE, the odd ones delta
+    auto issue_stat = [&](const float* src, int mb, float* dst) {
+        if (lane < BMI) {
+            int m = mb * BMI + lane;
+            m = m < M ? m : M - 1;
+            g2lds4_untracked(src, (unsigned)m * 4u, dst);
         }
-        if (ftid >= 256 - BMI)
-            reinterpret_cast<float*>(smem + C::OFF_DELTA)[(mb & (C::NDOB - 1)) * BMI + ftid - (256 - BMI)] = delta_r;
     };
-
-    // bias slice (BMI rows x 32 keys) of query block mb -> ring slot, straight from HBM to LDS.
-    // Chunk c = 64 it + lane of the slice (row c / BCPR, 16-byte chunk c % BCPR) lands at byte
-    // 16 c of the slot, i.e. the slot is the row-major slice.  Rows past M re-read row M - 1 and
-    // chunks that start past N re-read column 0: both are masked where they are used.  A block
-    // index past the end re-reads the last block, so that every step issues the same number of
-    // copies and their completion can be counted.
+    // bias slice (BMI rows x 32 keys) of query block mb -> ring slot.  Chunk c = 64 it + lane of the
+    // slice (row c / BCPR, 16-byte chunk c % BCPR) lands at byte 16 c of the slot, i.e. the slot
+    // is the row-major slice.  Rows past M re-read row M - 1 and chunks that start past N re-read
+    // column 0: both are masked where they are used.
     auto issue_bias = [&](int mb) {
         if constexpr (BIAS != 0) {
-            const int blk = mb < n_mblocks ? mb : n_mblocks - 1;
-            unsigned char* dst = ring_lds + ((mb - mb_first) & (C::RING - 1)) * C::BT_BYTES;
+            unsigned char* dst = ring_lds + ((mb - mb_first) % C::RING) * C::BT_BYTES;
 #pragma unroll
             for (int it = 0; it < C::BCH; it++) {
                 const int c = it * 64 + lane;
-                int m = blk * BMI + c / C::BCPR;
+                int m = mb * BMI + c / C::BCPR;
                 int nn = nw + (c % C::BCPR) * C::EPC;
                 m = m < M ? m : M - 1;
                 nn = nn < N ? nn : 0;
@@ -561,6 +544,20 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
             }
         }
     };
+    // block mb of Q with its LSE (QD + 1 copies) / block mb of dO with its delta (QD + 1 copies);
+    // all four waves of a role copy the 32 or 64 floats, which keeps their counts alike
+    auto issue_q = [&](int mb) {
+        issue_rows(qp, p.sq.s, cq_off, mb, smem + (mb % C::NQB) * C::Q_BYTES);
+        issue_stat(lsep, mb, reinterpret_cast<float*>(smem + C::OFF_LSE) + (mb % C::NQB) * BMI);
+    };
+    auto issue_do = [&](int mb) {
+        issue_rows(dop, p.sdo.s, cdo_off, mb, smem + C::OFF_DO + (mb % C::NDOB) * C::Q_BYTES);
+        issue_stat(deltap, mb, reinterpret_cast<float*>(smem + C::OFF_DELTA) + (mb % C::NDOB) * BMI);
+    };
+    // Issuing a copy stalls the wave while the memory pipeline of the CU is backed up, so the
+    // copies are dealt out to the role with less other work: Q goes with the S-waves, dO with the
+    // dP-waves unless those also write dBias.
+    constexpr bool Q_BY_S = true, DO_BY_S = DBIAS;
     // per-element path for bias rows that cannot be copied in aligned 16-byte chunks
     auto load_bias_scalar = [&](int mb, unsigned char* dst) {
         if constexpr (BIAS != 0) {
@@ -575,18 +572,14 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
         }
     };
 
-    // ---- prologue: Q(first) staged, Q(first+1) and dO(first) on their way ----
-    if (mb_first < n_mblocks) {
-        if (!s_wave) {
-            fetch_q(mb_first);
-            stage_q(mb_first);
-            fetch_q(mb_first + 1);
-            fetch_do(mb_first);
-        } else if (BIAS != 0 && bias_vec) {
+    // ---- prologue: the first LA blocks of Q and LA - 1 blocks of dO ----
 #pragma unroll 1
-            for (int mb = mb_first; mb < mb_first + C::RING - 1; mb++) issue_bias(mb);
-        }
+    for (int i = 0; i < C::LA; i++) {
+        if (s_wave == Q_BY_S) issue_q(mb_first + i);
+        if (s_wave && BIAS != 0 && bias_vec) issue_bias(mb_first + i);
+        if (s_wave == DO_BY_S && i < C::LA - 1) issue_do(mb_first + i);
     }
+    wait_vmcnt<0>();
     __syncthreads();
 
     T8 op_cur[NSUB][2];  // P^T (S-wave) or dS^T (dP-wave) of the block whose accumulation is still due
@@ -624,23 +617,22 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
 
     if (s_wave) {
         // ================================ S-wave ================================
+        auto s_loop = [&](auto bv_tag) {
+        constexpr bool BV = decltype(bv_tag)::value;                    // bias slices come by copy
+        constexpr int OPS = (BV ? C::BCH : 0) + ((Q_BY_S ? 1 : 0) + (DO_BY_S ? 1 : 0)) * (C::QD + 1);  // copies per step
 #pragma unroll 1
         for (int t = mb_first - 1; t <= n_mblocks; t++) {
             const int nb = t + 1;  // the block whose P is produced in this step
             T8 op_next[NSUB][2];
+            // copies for the steps to come; their buffers were last read one step ago
+            if constexpr (Q_BY_S) issue_q(nb + C::LA);
+            if constexpr (BV) issue_bias(nb + C::LA);
+            if constexpr (DO_BY_S) issue_do(t + C::LA);
             if (nb < n_mblocks) {
                 const int m0 = nb * BMI;
-                const unsigned char* bt_lds = ring_lds + ((nb - mb_first) & (C::RING - 1)) * C::BT_BYTES;
-                if constexpr (BIAS != 0) {
-                    if (bias_vec) {
-                        // the copies of block nb were issued RING - 1 steps ago and at most the
-                        // (RING - 2) * BCH copies issued since may still be in flight
-                        wait_vmcnt<(C::RING - 2) * C::BCH>();
-                        issue_bias(nb + C::RING - 1);  // into the slot the previous block has left
-                    } else {
-                        load_bias_scalar(nb, ring_lds + ((nb - mb_first) & (C::RING - 1)) * C::BT_BYTES);
-                    }
-                }
+                const unsigned char* bt_lds = ring_lds + ((nb - mb_first) % C::RING) * C::BT_BYTES;
+                if constexpr (BIAS != 0 && !BV)
+                    load_bias_scalar(nb, ring_lds + ((nb - mb_first) % C::RING) * C::BT_BYTES);
                 const bool need_mask = (m0 + BMI > M) || (n0 + BN > N) || (CAUSAL && m0 < n0 + BN - 1);
                 f32x16 sacc[NSUB];
                 gemm_rows(reinterpret_cast<const T*>(smem + (nb % C::NQB) * C::Q_BYTES), sacc);
@@ -703,13 +695,18 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
                 else p_step(std::false_type{});
             }
             if (t >= mb_first && t < n_mblocks)  // dV^T += dO(t)^T P(t)
-                gemm_cols(reinterpret_cast<const T*>(smem + C::OFF_DO + (t & (C::NDOB - 1)) * C::Q_BYTES), op_cur);
+                gemm_cols(reinterpret_cast<const T*>(smem + C::OFF_DO + (t % C::NDOB) * C::Q_BYTES), op_cur);
 #pragma unroll
             for (int sb = 0; sb < NSUB; sb++)
 #pragma unroll
                 for (int kk = 0; kk < 2; kk++) op_cur[sb][kk] = op_next[sb][kk];
+            // all copies but those of the last LA - 1 steps have landed; the barrier publishes them
+            wait_vmcnt<OPS*(C::LA - 1)>();
             lds_barrier();
         }
+        };
+        if (BIAS != 0 && bias_vec) s_loop(std::true_type{});
+        else s_loop(std::false_type{});
     } else {
         // ================================ dP-wave ================================
         T* ds_lds = reinterpret_cast<T*>(smem + C::OFF_DS);
@@ -731,21 +728,21 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
         }
         auto dp_loop = [&](auto fast_tag) {
         constexpr bool DB_FAST = decltype(fast_tag)::value;
+        // copies per step; the dBias stores that may sit between them in the queue are not
+        // counted, which only makes the wait at the end of a step stricter
+        constexpr int COPIES = ((Q_BY_S ? 0 : 1) + (DO_BY_S ? 0 : 1)) * (C::QD + 1);
 #pragma unroll 1
         for (int t = mb_first - 1; t <= n_mblocks; t++) {
-            // blocks on their way: Q(t+2), dO(t+1) registers -> LDS; Q(t+3), dO(t+2) -> registers
-            stage_q(t + 2);
-            stage_do(t + 1);
-            fetch_q(t + 3);
-            fetch_do(t + 2);
+            if constexpr (!Q_BY_S) issue_q(t + 1 + C::LA);
+            if constexpr (!DO_BY_S) issue_do(t + C::LA);
             if (C::DEFER_DK && t - 1 >= mb_first)  // dK^T += Q(t-1)^T dS(t-1)
                 gemm_cols(reinterpret_cast<const T*>(smem + ((t - 1) % C::NQB) * C::Q_BYTES), op_cur);
             if (t >= mb_first && t < n_mblocks) {
                 const int m0 = t * BMI;
                 f32x16 sacc[NSUB];
-                gemm_rows(reinterpret_cast<const T*>(smem + C::OFF_DO + (t & (C::NDOB - 1)) * C::Q_BYTES), sacc);
+                gemm_rows(reinterpret_cast<const T*>(smem + C::OFF_DO + (t % C::NDOB) * C::Q_BYTES), sacc);
                 // ---- dS = P (dP - delta) (flash_attention.py:303-308) ----
-                const float* delta_lds = reinterpret_cast<const float*>(smem + C::OFF_DELTA) + (t & (C::NDOB - 1)) * BMI;
+                const float* delta_lds = reinterpret_cast<const float*>(smem + C::OFF_DELTA) + (t % C::NDOB) * BMI;
                 const float* p_in = p_lds + (t & 1) * (C::P_BYTES / 4);
 #pragma unroll
                 for (int sb = 0; sb < NSUB; sb++) {
@@ -795,6 +792,7 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
                 if (!C::DEFER_DK)  // dK^T += Q(t)^T dS(t)
                     gemm_cols(reinterpret_cast<const T*>(smem + (t % C::NQB) * C::Q_BYTES), op_cur);
             }
+            if constexpr (COPIES > 0) wait_vmcnt<COPIES*(C::LA - 1)>();
             lds_barrier();
         }
         };

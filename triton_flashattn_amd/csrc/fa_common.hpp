@@ -157,6 +157,38 @@ __device__ __forceinline__ void g2lds16_untracked(const void* src, void* lds_bas
         : "v"(src), "s"(lds_addr)
         : "memory");
 }
+// The same with a wave-uniform base and a 32-bit byte offset per lane.
+__device__ __forceinline__ void g2lds16_untracked(const void* base, unsigned voff, void* lds_base) {
+    const unsigned lds_addr = __builtin_amdgcn_readfirstlane(
+        (unsigned)(uintptr_t)(__attribute__((address_space(3))) void*)lds_base);
+    unsigned saved_m0;
+    asm volatile(
+        "s_mov_b32 %0, m0\n\t"
+        "s_mov_b32 m0, %3\n\t"
+        "s_nop 0\n\t"
+        "global_load_lds_dwordx4 %1, %2\n\t"
+        "s_nop 0\n\t"
+        "s_mov_b32 m0, %0"
+        : "=&s"(saved_m0)
+        : "v"(voff), "s"(base), "s"(lds_addr)
+        : "memory");
+}
+// global_load_lds_dword: lane l copies the 4 bytes at base + voff (per lane) to lds_base + 4 l
+__device__ __forceinline__ void g2lds4_untracked(const void* base, unsigned voff, void* lds_base) {
+    const unsigned lds_addr = __builtin_amdgcn_readfirstlane(
+        (unsigned)(uintptr_t)(__attribute__((address_space(3))) void*)lds_base);
+    unsigned saved_m0;
+    asm volatile(
+        "s_mov_b32 %0, m0\n\t"
+        "s_mov_b32 m0, %3\n\t"
+        "s_nop 0\n\t"
+        "global_load_lds_dword %1, %2\n\t"
+        "s_nop 0\n\t"
+        "s_mov_b32 m0, %0"
+        : "=&s"(saved_m0)
+        : "v"(voff), "s"(base), "s"(lds_addr)
+        : "memory");
+}
 // s_waitcnt vmcnt(n) alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14, the other counters maxed)
 template <int N> __device__ __forceinline__ void wait_vmcnt() {
     __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));

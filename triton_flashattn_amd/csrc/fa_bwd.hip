@@ -356,7 +356,7 @@ template <int D, int BIAS> struct BwdCfg {
     static constexpr int DB = DP / 32;
     static constexpr int KSTEPS = D / 16;
     static constexpr int CPR = D / 8;
-    static constexpr int DSS = BN + 8;                     // dS tile row stride (elements)
+    static constexpr int DSS = BMI + 4;                    // dS^T tile: elements between two keys
     static constexpr int ES = BIAS == 0 ? 0 : (BIAS == 1 ? 1 : (BIAS == 4 ? 4 : 2));
     static constexpr int EPC = ES > 0 ? 16 / ES : 8;       // bias elements per 16-byte chunk
     static constexpr int BCPR = 2 * ES;                    // 16-byte chunks per 32-key bias row
@@ -367,7 +367,7 @@ template <int D, int BIAS> struct BwdCfg {
     // Q, dO, LSE, delta and the bias slices reach LDS through direct global -> LDS copies that the
     // S-waves issue LA blocks ahead of their use; a copy has LA - 1 whole steps and the rest of
     // its own to land before the barrier that publishes it.
-    static constexpr int DS_BYTES = (BIAS == 2 || BIAS == 3) ? BMI * DSS * 2 : 0;  // dS tile (dBias)
+    static constexpr int DS_BYTES = (BIAS == 2 || BIAS == 3) ? BN * DSS * 2 : 0;  // dS^T tiles (dBias)
     static constexpr int P_BYTES = 4 * NSUB * 64 * 64;     // P hand-off: 16 floats per lane per sub-block
     static constexpr int BT_BYTES = BMI * 32 * ES;         // bias slice of one S-wave
     // LDS bytes with copies la blocks ahead: la + 1 dO buffers and bias slots, la + 2 Q buffers and
@@ -555,9 +555,9 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
         issue_stat(deltap, mb, reinterpret_cast<float*>(smem + C::OFF_DELTA) + (mb % C::NDOB) * BMI);
     };
     // Issuing a copy stalls the wave while the memory pipeline of the CU is backed up, so the
-    // copies are dealt out to the role with less other work: Q goes with the S-waves, dO with the
-    // dP-waves unless those also write dBias.
-    constexpr bool Q_BY_S = true, DO_BY_S = DBIAS;
+    // copies are dealt out between the roles: Q and the bias go with the S-waves, dO with the
+    // dP-waves.
+    constexpr bool Q_BY_S = true, DO_BY_S = false;
     // per-element path for bias rows that cannot be copied in aligned 16-byte chunks
     auto load_bias_scalar = [&](int mb, unsigned char* dst) {
         if constexpr (BIAS != 0) {
@@ -628,6 +628,10 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
             if constexpr (Q_BY_S) issue_q(nb + C::LA);
             if constexpr (BV) issue_bias(nb + C::LA);
             if constexpr (DO_BY_S) issue_do(t + C::LA);
+            // dV^T += dO(t)^T P(t) first: its operands are ready, and the Q rows of the next block
+            // can be on their way out of LDS meanwhile
+            if (t >= mb_first && t < n_mblocks)
+                gemm_cols(reinterpret_cast<const T*>(smem + C::OFF_DO + (t % C::NDOB) * C::Q_BYTES), op_cur);
             if (nb < n_mblocks) {
                 const int m0 = nb * BMI;
                 const unsigned char* bt_lds = ring_lds + ((nb - mb_first) % C::RING) * C::BT_BYTES;
@@ -694,8 +698,6 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
                 if (need_mask) p_step(std::true_type{});
                 else p_step(std::false_type{});
             }
-            if (t >= mb_first && t < n_mblocks)  // dV^T += dO(t)^T P(t)
-                gemm_cols(reinterpret_cast<const T*>(smem + C::OFF_DO + (t % C::NDOB) * C::Q_BYTES), op_cur);
 #pragma unroll
             for (int sb = 0; sb < NSUB; sb++)
 #pragma unroll
@@ -709,21 +711,26 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
         else s_loop(std::false_type{});
     } else {
         // ================================ dP-wave ================================
-        T* ds_lds = reinterpret_cast<T*>(smem + C::OFF_DS);
+        // dS^T tile of this wave: 32 keys x BMI rows.  A lane writes its 4 consecutive rows of one key
+        // with one 8-byte store, and ds_read_b64_tr_b16 hands a lane 4 consecutive keys of one row.
+        T* ds_lds = reinterpret_cast<T*>(smem + C::OFF_DS) + kb * 32 * DSS;
+        static_assert(!DB_VIA_LDS || BMI == 32, "the dBias path is laid out for 32-row blocks");
+        // lane -> row 16 ((lane/16)%2) + lane%16, keys 8 (lane/32 + 2 it) .. + 7 of the slice
+        const int db_row = 16 * ((lane >> 4) & 1) + (lane & 15);
+        const int db_src = (8 * (lane >> 5) + ((lane & 15) >> 2)) * DSS + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
         // dBias rows that are whole aligned 16-byte chunks leave through unconditional buffer
         // stores (chunks outside the tensor get an offset outside the view): a loop without
         // branches around its stores lets the loads of the next blocks stay in flight across them.
         const bool db_fast = DB_VIA_LDS && dbias_vec && (N % 8 == 0);
         __amdgpu_buffer_rsrc_t db_rsrc = make_buffer(nullptr, 0);
-        int db_off[(BMI * 4) / 64];
+        int db_off[2];
         const int db_row_bytes = DB_VIA_LDS ? (int)p.sdbias.m * 2 : 0;
         if (db_fast) {
             db_rsrc = make_buffer(dbp, ((int64_t)(M - 1) * p.sdbias.m + N) * 2);
 #pragma unroll
-            for (int it = 0; it < (BMI * 4) / 64; it++) {
-                const int c = it * 64 + lane;
-                const int nn = nw + (c & 3) * 8;
-                db_off[it] = nn < N ? (c >> 2) * db_row_bytes + nn * 2 : (int)0x80000000;
+            for (int it = 0; it < 2; it++) {
+                const int nn = nw + 8 * ((lane >> 5) + 2 * it);
+                db_off[it] = nn < N ? db_row * db_row_bytes + nn * 2 : (int)0x80000000;
             }
         }
         auto dp_loop = [&](auto fast_tag) {
@@ -751,40 +758,44 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
                         const int ml0 = sb * 32 + 8 * q4 + 4 * g;
                         const f32x4 del4 = *reinterpret_cast<const f32x4*>(delta_lds + ml0);
                         const f32x4 p4 = *reinterpret_cast<const f32x4*>(p_in + ((sb * 4 + q4) * 64 + lane) * 4);
+                        T4 d4;
 #pragma unroll
                         for (int e = 0; e < 4; e++) {
                             const int i = q4 * 4 + e;
                             const float dsv = p4[e] * (sacc[sb][i] - del4[e]);
                             op_cur[sb][i >> 3][i & 7] = (T)dsv;
-                            if constexpr (DB_VIA_LDS) ds_lds[(ml0 + e) * DSS + kb * 32 + r] = (T)dsv;
+                            d4[e] = (T)dsv;
                             if constexpr (DBIAS && !DB_VIA_LDS) {
                                 const int m = m0 + ml0 + e;
                                 if (m < M && my_n < N) dbp[(int64_t)m * p.sdbias.m + (int64_t)my_n * p.sdbias.n] = (E)dsv;
                             }
                         }
+                        if constexpr (DB_VIA_LDS) *reinterpret_cast<T4*>(ds_lds + r * DSS + ml0) = d4;
                     }
                 }
-                // ---- dBias rows of this wave's 32 keys, 16 bytes per lane, out of the dS tile ----
+                // ---- dBias rows of this wave's 32 keys, 16 bytes per lane, out of the dS^T tile ----
                 if constexpr (DB_VIA_LDS) {
 #pragma unroll
-                    for (int it = 0; it < (BMI * 4) / 64; it++) {
-                        const int c = it * 64 + lane;
-                        const int row = c >> 2, ch = c & 3;
-                        const int m = m0 + row, nn = nw + ch * 8;
+                    for (int it = 0; it < 2; it++) {
+                        const i16x4 lo = lds_read_tr4(ds_lds + db_src + it * 16 * DSS);
+                        const i16x4 hi = lds_read_tr4(ds_lds + db_src + it * 16 * DSS + 4 * DSS);
+                        typedef short i16x8 __attribute__((ext_vector_type(8)));
+                        const i32x4 v = __builtin_bit_cast(i32x4, (i16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+                        const int m = m0 + db_row, nn = nw + 8 * ((lane >> 5) + 2 * it);
                         if constexpr (DB_FAST) {
-                            const T* src = ds_lds + row * DSS + kb * 32 + ch * 8;
                             // rows past M: m0 * row bytes alone is past the view only if the view is
                             // tight, so the row test is explicit
                             const int off = m < M ? db_off[it] + m0 * db_row_bytes : (int)0x80000000;
-                            buf_store16(db_rsrc, lds_read16(src), off);
+                            buf_store16(db_rsrc, v, off);
                         } else if (m < M && nn < N) {
-                            const T* src = ds_lds + row * DSS + kb * 32 + ch * 8;
                             E* dst = dbp + (int64_t)m * p.sdbias.m + (int64_t)nn * p.sdbias.n;
                             if (dbias_vec && nn + 8 <= N) {
-                                gst16(dst, lds_read16(src));
+                                gst16(dst, v);
                             } else {
+                                const T8 v8 = as_vec<T8>(v);
+#pragma unroll
                                 for (int e = 0; e < 8; e++)
-                                    if (nn + e < N) dst[(int64_t)e * p.sdbias.n] = __builtin_bit_cast(E, src[e]);
+                                    if (nn + e < N) dst[(int64_t)e * p.sdbias.n] = __builtin_bit_cast(E, (T)v8[e]);
                             }
                         }
                     }

@@ -23,6 +23,10 @@ import torch
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, GB/s
 MFMA_PEAK_TFLOPS = 2516.6    # MI355X dense bf16/fp16 MFMA, TFLOP/s
+# HBM bytes per launch of the roofline kernel on the headline workload: rocprofv3 FETCH_SIZE and
+# WRITE_SIZE, each scaled by what the same counter reads for a plain 1 GiB copy
+# (profiles/fa_kernels_c3_hbm_traffic.txt: 1.209 GB read + 1.141 GB written)
+ROOFLINE_KERNEL_TRAFFIC_BYTES = 2.350e9
 
 
 def log(*a):
@@ -239,7 +243,7 @@ def main():
         "roofline": {
             "kernel": "fa_bwd_kernel<bf16, D=128, bias=bf16, non-causal, dbias>",
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+            "frac": achieved / HBM_PEAK_GBS, "traffic": ROOFLINE_KERNEL_TRAFFIC_BYTES,
             "algorithmic_bytes_per_launch": y_main, "avg_launch_ms": t_main,
             # the kernel's own share of the algorithmic backward FLOPs: 4 of the 5 matrix products
             "mfma_frac_same_kernel": 0.8 * f_bwd / (t_main * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS,

@@ -63,6 +63,8 @@ bool bias_vec_ok(const void* ptr, const int64_t s[4], const fa_problem& p) {
     if (p.B > 1 && (s[0] * es) % 16 != 0) return false;
     if (p.H > 1 && (s[1] * es) % 16 != 0) return false;
     if (p.M > 1 && (s[2] * es) % 16 != 0) return false;
+    // whole 16-byte chunks only: a copy never reads past the end of a row
+    if (((int64_t)p.N * es) % 16 != 0) return false;
     // one (batch, head) slice is addressed through a 32-bit buffer descriptor
     if (s[2] < 0 || ((int64_t)(p.M - 1) * s[2] + p.N) * es >= (1ll << 31)) return false;
     return true;

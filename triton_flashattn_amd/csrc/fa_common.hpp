@@ -255,6 +255,45 @@ template <int D, int BIAS> struct RowCfg {
     static constexpr int MIN_BLOCKS = D <= 128 ? 2 : 1;
 };
 
+// Tiling of the forward kernel: a work-group owns 128 query rows (4 waves x 32 rows) and streams
+// keys in steps of NH blocks of 32.  K and V rows of a step and the bias slice of each wave reach
+// LDS through direct global -> LDS copies issued ahead of their use.  With a bias: steps of 32
+// keys, K/V in a ring of 3 slots (two steps ahead), the bias in a ring of 4 slots per wave (three
+// steps ahead).  Without: steps of 64 keys, K/V double buffered (one step ahead), which halves the
+// number of barriers.
+template <int D, int BIAS> struct StreamCfg {
+    static constexpr int NH = BIAS == 0 ? 2 : 1;     // 32-key blocks per step
+    static constexpr int LA = BIAS == 0 ? 1 : 2;     // steps the K/V copies run ahead
+    static constexpr int BM = 128, BK = 32 * NH, NT = 256;
+    static constexpr int DP = D < 32 ? 32 : D;       // head dim padded to one 32-wide MFMA block
+    static constexpr int OS = DP + 8;                // O staging row stride (elements)
+    static constexpr int CPR = D / 8;                // 16-byte chunks per row
+    static constexpr int KSTEPS = D / 16;            // MFMA k-steps of Q K^T
+    static constexpr int DB = DP / 32;               // 32-wide blocks of the head dim
+    static constexpr int ES = BIAS == 0 ? 0 : (BIAS == 1 ? 1 : (BIAS == 4 ? 4 : 2));
+    static constexpr int EPC = ES > 0 ? 16 / ES : 8; // bias elements per 16-byte chunk
+    static constexpr int STEP_BYTES = BK * D * 2;    // K (or V) rows of one step, unpadded, swizzled
+    static constexpr int NKD = STEP_BYTES / 1024;    // 1 KB copies per K (or V) step
+    static constexpr int KD = NKD >= 4 ? NKD / 4 : 1;  // of which each wave issues this many
+    static constexpr int NKV = LA + 1;               // K/V ring slots
+    static constexpr int O_BYTES = BM * OS * 2;
+    static constexpr int KV_BYTES = 2 * NKV * STEP_BYTES > O_BYTES ? 2 * NKV * STEP_BYTES : O_BYTES;
+    static constexpr int BCPR = 2 * ES;              // 16-byte chunks per bias row of 32 keys
+    static constexpr int BROW = 32 * ES;             // bytes per bias row of a slot
+    static constexpr int BSLOT = 32 * BROW;          // one wave's bias slice of one step
+    static constexpr int BCH = BSLOT / 1024;         // 1 KB copies per bias slice
+    static constexpr int NBS = 4;                    // bias ring slots per wave
+    static constexpr int BIAS_BYTES = 4 * NBS * BSLOT;
+    static constexpr int LDS_BYTES = KV_BYTES + BIAS_BYTES;
+    // 16-byte chunk c of bias row `row` is stored at chunk c ^ bswz(row): rows that share LDS banks
+    // get different chunk orders
+    __device__ static __forceinline__ int bswz(int row) {
+        return ES == 4 ? ((row >> 1) & 7) : (ES == 2 ? ((row >> 2) & 3) : ((row >> 3) & 1));
+    }
+    // two work-groups per CU whenever registers and LDS allow it
+    static constexpr int MIN_BLOCKS = (D <= 128 && LDS_BYTES <= 81920) ? 2 : 1;
+};
+
 // Work-group id -> (tile, batch*head).  Work-groups are dealt round-robin to the 8 XCDs; when
 // the number of (batch, head) pairs is a multiple of 8 every tile of one pair is sent to the same
 // XCD so that its K/V (or Q/dO) stay in that XCD's L2.

@@ -5,15 +5,20 @@
 // the kernel as an fp32 multiply.
 //
 // Work split.  One work-group (4 waves) owns 128 query rows of one (batch, head); each wave
-// owns 32 of them for the whole kernel.  Keys/values are streamed in tiles of 64 through LDS.
+// owns 32 of them for the whole kernel.  Keys/values are streamed through LDS in steps of 32
+// (with a bias) or 64 keys, consumed 32 at a time.
 // Scores are computed TRANSPOSED, S^T = K Q^T, so that in the MFMA accumulator a lane holds one
-// query row (column l%32 of S^T) and 32 of the 64 keys: the row maximum and row sum of the online
+// query row (column l%32 of S^T) and 16 of the 32 keys: the row maximum and row sum of the online
 // softmax are then per-lane loops plus a single exchange with lane l^32, the running maximum, the
 // running sum and the rescale factor are one scalar per lane, and P^T is already laid out as the
-// B operand of O^T += V^T P^T.  V^T is gathered from the row-major V tile with
-// ds_read_b64_tr_b16.  The bias tile of a wave (32 rows x 64 keys) is staged through a
-// wave-private LDS region with 16-byte coalesced global loads and read back in accumulator
-// layout (4 consecutive keys per read).
+// B operand of O^T += V^T P^T.  V^T is gathered from the row-major V rows with
+// ds_read_b64_tr_b16.
+//
+// Memory -> LDS.  The K and V rows of a step (ring of 3 slots issued two steps ahead; double
+// buffered and one step ahead without a bias) and the bias slice of each wave (32 rows x 32 keys,
+// ring of 4 wave-private slots, issued three steps ahead) arrive through direct global -> LDS copies that the compiler does not see; their
+// completion is counted by hand (copies complete in issue order and every step issues the same
+// number).  The bias is a pure HBM stream: only a queue this deep keeps enough bytes in flight.
 #include <type_traits>
 
 #include "fa_common.hpp"
@@ -22,13 +27,13 @@
 namespace fa {
 
 template <typename T, int D, int BIAS, bool CAUSAL>
-__global__ __launch_bounds__(256, (RowCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_kernel(const FwdParams p) {
-    typedef RowCfg<D, BIAS> C;
+__global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_kernel(const FwdParams p) {
+    typedef StreamCfg<D, BIAS> C;
     typedef Swz<D> SW;
     typedef typename VecOf<T>::v8 T8;
     typedef typename VecOf<T>::v4 T4;
     typedef typename BiasElem<BIAS>::type E;
-    constexpr int BM = C::BM, BN = C::BN, OS = C::OS, CPR = C::CPR;
+    constexpr int BM = C::BM, BK = C::BK, OS = C::OS, CPR = C::CPR;
 
     __shared__ __align__(16) unsigned char smem[C::LDS_BYTES];
 
@@ -46,13 +51,13 @@ __global__ __launch_bounds__(256, (RowCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_ker
     const int my_m = mw + r;
 
     const T* qp = reinterpret_cast<const T*>(p.q) + (int64_t)b * p.sq.b + (int64_t)h * p.sq.h;
-    const char* kbase = reinterpret_cast<const char*>(reinterpret_cast<const T*>(p.k) + (int64_t)b * p.sk.b + (int64_t)h * p.sk.h);
-    const char* vbase = reinterpret_cast<const char*>(reinterpret_cast<const T*>(p.v) + (int64_t)b * p.sv.b + (int64_t)h * p.sv.h);
+    const T* kp = reinterpret_cast<const T*>(p.k) + (int64_t)b * p.sk.b + (int64_t)h * p.sk.h;
+    const T* vp = reinterpret_cast<const T*>(p.v) + (int64_t)b * p.sv.b + (int64_t)h * p.sv.h;
     const E* bp = nullptr;
-    unsigned char* bias_lds = nullptr;
+    unsigned char* bias_lds = nullptr;  // this wave's ring of bias slots
     if (BIAS != 0) {
         bp = reinterpret_cast<const E*>(p.bias) + (int64_t)b * p.sbias.b + (int64_t)h * p.sbias.h;
-        bias_lds = smem + C::KV_BYTES + wave * 32 * C::BROW;
+        bias_lds = smem + C::KV_BYTES + wave * C::NBS * C::BSLOT;
     }
 
     // Q^T as B operand: column my_m, k = d
@@ -64,10 +69,10 @@ __global__ __launch_bounds__(256, (RowCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_ker
         qreg[ks] = as_vec<T8>(raw);
     }
 
-    int n_tiles = (N + BN - 1) / BN;
+    int n_steps = (N + BK - 1) / BK;
     if (CAUSAL) {
-        int last = (m0 + BM - 1) / BN + 1;  // tiles holding keys <= last row of this work-group
-        n_tiles = n_tiles < last ? n_tiles : last;
+        int last = (m0 + BM - 1) / BK + 1;  // steps holding keys <= last row of this work-group
+        n_steps = n_steps < last ? n_steps : last;
     }
 
     const float qk_scale = p.sm_scale * kLog2e;
@@ -78,249 +83,249 @@ __global__ __launch_bounds__(256, (RowCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_ker
 #pragma unroll
         for (int i = 0; i < 16; i++) o_acc[db][i] = 0.f;
 
-    // ---- K / V tiles: global -> LDS without passing through registers.  Chunk c of a tile
-    // (row c / CPR, LDS chunk c % CPR) is copied by thread c % 256 in copy c / 256; the LDS chunk
-    // holds global chunk (c % CPR) ^ f(row), which is the swizzle the readers expect.
-    unsigned koff[C::NCH], voff[C::NCH];  // byte offsets of this lane's source chunks in a full tile
+    // ---- K / V rows of a step: NKD copies of 1 KB each; copy ci fills bytes [1024 ci, 1024 ci + 1024)
+    // of the swizzled slot, so lane l of it fetches the chunk that lives at slot position 64 ci + l
+    // (row c / CPR, LDS chunk c % CPR holds global chunk (c % CPR) ^ f(row)).  Each wave issues KD
+    // of them (more than once where a step has fewer than four).  Rows past N re-read row N - 1:
+    // their scores are masked.
+    unsigned k_off[C::KD], v_off[C::KD];
+    int c_idx[C::KD];
 #pragma unroll
-    for (int it = 0; it < C::NCH; it++) {
-        const int c = it * C::NT + tid;
+    for (int i = 0; i < C::KD; i++) {
+        c_idx[i] = (wave * C::KD + i) % C::NKD;
+        const int c = c_idx[i] * 64 + lane;
         const int row = c / CPR, src = (c % CPR) ^ SW::f(row);
-        koff[it] = (unsigned)(row * (int)p.sk.s * 2 + src * 16);
-        voff[it] = (unsigned)(row * (int)p.sv.s * 2 + src * 16);
+        k_off[i] = (unsigned)(row * (int)p.sk.s * 2 + src * 16);
+        v_off[i] = (unsigned)(row * (int)p.sv.s * 2 + src * 16);
     }
-    auto issue_tile = [&](int j, int buf) {
-        const int n0 = j * BN;
-        const char* kt = kbase + (int64_t)n0 * p.sk.s * 2;
-        const char* vt = vbase + (int64_t)n0 * p.sv.s * 2;
-        unsigned char* k_dst = smem + buf * C::TILE_BYTES;
-        unsigned char* v_dst = smem + (2 + buf) * C::TILE_BYTES;
-        const bool full = n0 + BN <= N;
+    auto issue_kv = [&](int k) {
+        const int n0 = k * BK < N ? k * BK : N - 1;  // a step past the end is the last row over and over
+        const T* kt = kp + (int64_t)n0 * p.sk.s;
+        const T* vt = vp + (int64_t)n0 * p.sv.s;
+        unsigned char* k_dst = smem + (k % C::NKV) * C::STEP_BYTES;
+        unsigned char* v_dst = smem + (C::NKV + k % C::NKV) * C::STEP_BYTES;
+        const bool full = n0 + BK <= N;
 #pragma unroll
-        for (int it = 0; it < C::NCH; it++) {
-            const int c0 = it * C::NT + wave * 64;  // first chunk of this wave's copy
-            if (c0 < C::TILE_CHUNKS) {
-                unsigned ko = koff[it], vo = voff[it];
-                if (!full) {  // rows past the last key re-read the last key; the scores are masked
-                    const int c = c0 + lane;
-                    int row = c / CPR;
-                    const int src = (c % CPR) ^ SW::f(row);
-                    row = row < N - n0 ? row : N - n0 - 1;
-                    ko = (unsigned)(row * (int)p.sk.s * 2 + src * 16);
-                    vo = (unsigned)(row * (int)p.sv.s * 2 + src * 16);
-                }
-                g2lds16(kt + ko, k_dst + c0 * 16);
-                g2lds16(vt + vo, v_dst + c0 * 16);
+        for (int i = 0; i < C::KD; i++) {
+            unsigned ko = k_off[i], vo = v_off[i];
+            if (!full) {
+                const int c = c_idx[i] * 64 + lane;
+                int row = c / CPR;
+                const int src = (c % CPR) ^ SW::f(row);
+                row = row < N - n0 ? row : N - 1 - n0;
+                ko = (unsigned)(row * (int)p.sk.s * 2 + src * 16);
+                vo = (unsigned)(row * (int)p.sv.s * 2 + src * 16);
+            }
+            g2lds16_untracked(kt, ko, k_dst + c_idx[i] * 1024);
+            g2lds16_untracked(vt, vo, v_dst + c_idx[i] * 1024);
+        }
+    };
+    // ---- bias slice of this wave for step k (32 rows x 32 keys) -> ring slot k % NBS.  Position c =
+    // 64 it + lane of the slot (row c / BCPR, LDS chunk c % BCPR) holds chunk (c % BCPR) ^ bswz(row)
+    // of the row.  Rows past M re-read row M - 1 (never stored) and chunks that start past N
+    // re-read column 0 (masked).
+    auto issue_bias = [&](int k) {
+        if constexpr (BIAS != 0) {
+            unsigned char* dst = bias_lds + (k % C::NBS) * C::BSLOT;
+#pragma unroll
+            for (int it = 0; it < C::BCH; it++) {
+                const int c = it * 64 + lane;
+                const int row = c / C::BCPR;
+                int m = mw + row;
+                int n = k * BK + ((c % C::BCPR) ^ C::bswz(row)) * C::EPC;
+                m = m < M ? m : M - 1;
+                n = n < N ? n : 0;
+                g2lds16_untracked(bp + (int64_t)m * p.sbias.m + n, dst + it * 1024);
             }
         }
     };
 
-    // ---- bias tile of this wave (32 rows x 64 keys): global -> registers one tile ahead ----
-    i32x4 breg[C::BCH > 0 ? C::BCH : 1];
-    int boff[C::BCH > 0 ? C::BCH : 1];
-    __amdgpu_buffer_rsrc_t brsrc = make_buffer(nullptr, 0);
-    if constexpr (BIAS != 0) {
-        constexpr int CH_ROW = 4 * C::ES;  // 16-byte chunks per 64-key row
-#pragma unroll
-        for (int it = 0; it < C::BCH; it++) {
-            const int c = it * 64 + lane;
-            boff[it] = (c / CH_ROW) * (int)p.sbias.m * C::ES + (c % CH_ROW) * 16;
-        }
-        // everything from the first row of this wave to the end of the (b, h) slice
-        brsrc = make_buffer(bp + (int64_t)mw * p.sbias.m, ((int64_t)(M - 1 - mw) * p.sbias.m + N) * C::ES);
-    }
-    auto prefetch_bias = [&](int j) {
-        if constexpr (BIAS != 0) {
-            if (p.bias_vec) {
-#pragma unroll
-                for (int it = 0; it < C::BCH; it++) breg[it] = buf_load16(brsrc, boff[it], j * BN * C::ES);
-            }
-        }
-    };
-
-    if (n_tiles > 0) {
-        issue_tile(0, 0);
-        prefetch_bias(0);
-    }
-
-    // One tile of the K/V stream.  Interior tiles (every key in range and visible to every row of
-    // the work-group) run with TILE_MASKED = false: no range checks, no mask arithmetic.
-    auto tile_step = [&](int j, auto tile_tag) {
-        constexpr bool TILE_MASKED = decltype(tile_tag)::value;
-        const int n0 = j * BN;
-        const int buf = j & 1;
-        const T* k_lds = reinterpret_cast<const T*>(smem + buf * C::TILE_BYTES);
-        const T* v_lds = reinterpret_cast<const T*>(smem + (2 + buf) * C::TILE_BYTES);
-        __builtin_amdgcn_s_waitcnt(0);  // this thread's copies of tile j (and its bias chunks) have landed
-        if constexpr (BIAS != 0) {
-            if (p.bias_vec) {
-#pragma unroll
-                for (int it = 0; it < C::BCH; it++) {
-                    constexpr int CH_ROW = 4 * C::ES;
-                    const int c = it * 64 + lane;
-                    const int row = c / CH_ROW;
-                    lds_write16(bias_lds + row * C::BROW + (((c % CH_ROW) ^ C::bswz(row)) << 4), breg[it]);
-                }
-            } else {
-                // unaligned bias rows or non-unit key stride: one element per lane per row
+    // One step of the K/V stream.  Interior steps (every key in range and visible to every row of
+    // the work-group) run with STEP_MASKED = false: no range checks, no mask arithmetic.  BV: the
+    // bias slices come by copy (rows that allow aligned 16-byte chunks), else element by element.
+    auto kv_step = [&](int k, auto step_tag, auto bv_tag) {
+        constexpr bool STEP_MASKED = decltype(step_tag)::value;
+        constexpr bool BV = decltype(bv_tag)::value;
+        constexpr int OPS = 2 * C::KD + (BV ? C::BCH : 0);  // copies per wave per step
+        const int n0 = k * BK;
+        const T* k_lds = reinterpret_cast<const T*>(smem + (k % C::NKV) * C::STEP_BYTES);
+        const T* v_lds = reinterpret_cast<const T*>(smem + (C::NKV + k % C::NKV) * C::STEP_BYTES);
+        const unsigned char* b_lds = bias_lds + (k % C::NBS) * C::BSLOT;
+        // K/V of this step were issued LA steps ago; the bias copies issued right after them and
+        // the copies of the steps since may still be in flight
+        wait_vmcnt<(BV ? C::BCH : 0) + OPS*(C::LA - 1)>();
+        lds_barrier();  // step k is complete in LDS; nobody still reads the slot of step k - 1
+        issue_kv(k + C::LA);
+        if constexpr (BV) issue_bias(k + C::NBS - 1);
+        if constexpr (BIAS != 0 && !BV) {
+            // unaligned bias rows or non-unit key stride: one element per lane per row
+            if (lane < 32) {
 #pragma unroll 1
                 for (int row = 0; row < 32; row++) {
-                    int n = n0 + lane;
+                    const int n = n0 + lane;
                     E val = (E)0.f;
-                    if (mw + row < M && n < N)
-                        val = bp[(int64_t)(mw + row) * p.sbias.m + (int64_t)n * p.sbias.n];
+                    if (mw + row < M && n < N) val = bp[(int64_t)(mw + row) * p.sbias.m + (int64_t)n * p.sbias.n];
                     const int byte = lane * C::ES;
-                    *reinterpret_cast<E*>(bias_lds + row * C::BROW + (((byte >> 4) ^ C::bswz(row)) << 4) + (byte & 15)) = val;
+                    *reinterpret_cast<E*>(bias_lds + (k % C::NBS) * C::BSLOT + row * C::BROW + (((byte >> 4) ^ C::bswz(row)) << 4) + (byte & 15)) = val;
                 }
             }
         }
-        __syncthreads();  // tile j is complete in LDS; nobody still reads the buffer of tile j - 1
-        if (j + 1 < n_tiles) {
-            issue_tile(j + 1, buf ^ 1);
-            prefetch_bias(j + 1);
+        static_assert(BIAS == 0 || C::NH == 1, "a bias slot covers one 32-key block");
+        // The step is consumed 32 keys at a time, each block with its own softmax step, so that only
+        // one 32 x 32 score block is live at a time.
+#pragma unroll
+        for (int nb = 0; nb < C::NH; nb++) {
+        const int nh = nb * 32;  // first key of this block inside the step
+        __builtin_amdgcn_sched_barrier(0);  // keep the blocks apart
+        // blocks entirely above this wave's diagonal or past the last key contribute nothing
+        if (STEP_MASKED && ((CAUSAL && n0 + nh > mw + 31) || n0 + nh >= N)) continue;
+        const bool need_mask = STEP_MASKED && ((n0 + nh + 32 > N) || (CAUSAL && n0 + nh + 31 > mw));
+
+        // ---- S^T = K Q^T : s[i] is key n0 + nh + 8 (i/4) + 4 g + i%4, query my_m ----
+        f32x16 s;
+#pragma unroll
+        for (int i = 0; i < 16; i++) s[i] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < C::KSTEPS; ks++) {
+            T8 a = as_vec<T8>(lds_read16(k_lds + SW::off(nh + r, ks * 16 + 8 * g)));
+            s = mfma32(a, qreg[ks], s);
         }
 
-        // The 64-key tile is consumed as two 32-key halves, each with its own softmax step, so
-        // that only one 32 x 32 score block is live at a time.
+        // ---- online softmax step.  `masked` steps (ragged edge, causal diagonal) and a
+        // non-positive scale follow the reference's arithmetic term by term: scaled score,
+        // plus additive -1e6 terms in log2 units, plus bias (flash_attention.py:39-53).  Interior
+        // steps skip the mask terms and fold the scale into the exponent.
+        // The running maximum m_i is only raised when a step exceeds it by more than 2^8: the
+        // reference point of the exponentials is arbitrary (out = acc / l and LSE = m + log2 l
+        // do not depend on it), so a stale one costs nothing but saves rescaling O every step.
+        T8 pb[2];
+        auto softmax_step = [&](auto masked_tag) {
+            constexpr bool MASKED = decltype(masked_tag)::value;
+            float mx = -INFINITY;
 #pragma unroll
-        for (int nb = 0; nb < 2; nb++) {
-            const int nh = nb * 32;  // first key of this half inside the tile
-            __builtin_amdgcn_sched_barrier(0);  // keep the halves apart: one score block live at a time
-            // halves entirely above this wave's diagonal contribute nothing
-            if (TILE_MASKED && CAUSAL && n0 + nh > mw + 31) continue;
-            if (TILE_MASKED && n0 + nh >= N) continue;
-            const bool need_mask = TILE_MASKED && ((n0 + nh + 32 > N) || (CAUSAL && n0 + nh + 31 > mw));
-
-            // ---- S^T = K Q^T : s[i] is key n0 + nh + 8 (i/4) + 4 g + i%4, query my_m ----
-            f32x16 s;
+            for (int q4 = 0; q4 < 4; q4++) {
+                const int nl = 8 * q4 + 4 * g;            // first of 4 consecutive keys
+                const int byte = nl * C::ES;              // where they start in the bias row
+                float bv[4] = {0.f, 0.f, 0.f, 0.f};       // bias in natural units
+                bool keep[4] = {true, true, true, true};
+                if constexpr (BIAS == 1) {
+                    unsigned int w = *reinterpret_cast<const unsigned int*>(b_lds + r * C::BROW + (((byte >> 4) ^ C::bswz(r)) << 4) + (byte & 15));
 #pragma unroll
-            for (int i = 0; i < 16; i++) s[i] = 0.f;
+                    for (int e = 0; e < 4; e++) keep[e] = ((w >> (8 * e)) & 0xffu) != 0;
+                } else if constexpr (BIAS == 2 || BIAS == 3) {
+                    typedef typename VecOf<E>::v4 B4;
+                    B4 hv = *reinterpret_cast<const B4*>(b_lds + r * C::BROW + (((byte >> 4) ^ C::bswz(r)) << 4) + (byte & 15));
 #pragma unroll
-            for (int ks = 0; ks < C::KSTEPS; ks++) {
-                T8 a = as_vec<T8>(lds_read16(k_lds + SW::off(nh + r, ks * 16 + 8 * g)));
-                s = mfma32(a, qreg[ks], s);
-            }
-
-            // ---- online softmax step.  `masked` tiles (ragged edge, causal diagonal) and a
-            // non-positive scale follow the reference's arithmetic term by term: scaled score,
-            // plus additive -1e6 terms in log2 units, plus bias (flash_attention.py:39-53).  Interior
-            // tiles skip the mask terms and fold the scale into the exponent.
-            // The running maximum m_i is only raised when a tile exceeds it by more than 2^8: the
-            // reference point of the exponentials is arbitrary (out = acc / l and LSE = m + log2 l
-            // do not depend on it), so a stale one costs nothing but saves rescaling O every tile.
-            T8 pb[2];
-            auto softmax_step = [&](auto masked_tag) {
-                constexpr bool MASKED = decltype(masked_tag)::value;
-                float mx = -INFINITY;
-                {
+                    for (int e = 0; e < 4; e++) bv[e] = (float)hv[e];
+                } else if constexpr (BIAS == 4) {
+                    f32x4 w = *reinterpret_cast<const f32x4*>(b_lds + r * C::BROW + (((byte >> 4) ^ C::bswz(r)) << 4));
 #pragma unroll
-                    for (int q4 = 0; q4 < 4; q4++) {
-                        const int nl = nh + 8 * q4 + 4 * g;  // first of 4 consecutive keys
-                        float bv[4] = {0.f, 0.f, 0.f, 0.f};       // bias in natural units
-                        bool keep[4] = {true, true, true, true};
-                        if constexpr (BIAS == 1) {
-                            unsigned int w = *reinterpret_cast<const unsigned int*>(bias_lds + r * C::BROW + (((nl >> 4) ^ C::bswz(r)) << 4) + (nl & 15));
+                    for (int e = 0; e < 4; e++) bv[e] = w[e];
+                }
 #pragma unroll
-                            for (int e = 0; e < 4; e++) keep[e] = ((w >> (8 * e)) & 0xffu) != 0;
-                        } else if constexpr (BIAS == 2 || BIAS == 3) {
-                            typedef typename VecOf<E>::v4 B4;
-                            B4 hv = *reinterpret_cast<const B4*>(bias_lds + r * C::BROW + (((nl >> 3) ^ C::bswz(r)) << 4) + ((nl * 2) & 15));
-#pragma unroll
-                            for (int e = 0; e < 4; e++) bv[e] = (float)hv[e];
-                        } else if constexpr (BIAS == 4) {
-                            f32x4 w = *reinterpret_cast<const f32x4*>(bias_lds + r * C::BROW + (((nl >> 2) ^ C::bswz(r)) << 4));
-#pragma unroll
-                            for (int e = 0; e < 4; e++) bv[e] = w[e];
-                        }
-#pragma unroll
-                        for (int e = 0; e < 4; e++) {
-                            const int i = q4 * 4 + e;
-                            float x;
-                            if constexpr (MASKED) {
-                                x = __fmul_rn(s[i], qk_scale);
-                                const int n = n0 + nl + e;
-                                float t = (n >= N) ? kMask : 0.f;
-                                if (CAUSAL) t += (my_m < n) ? kMask : 0.f;
-                                float add = 0.f;
-                                if (BIAS == 1) add = keep[e] ? 0.f : kMask;
-                                if (BIAS >= 2) add = __fmul_rn(bv[e], kLog2e);
-                                if (BIAS != 0) add = (n >= N) ? kMask : add;  // out-of-range bias reads as masked
-                                x = __fadd_rn(x, __fadd_rn(t, add));
-                            } else if constexpr (BIAS == 0) {
-                                x = s[i];                                    // raw score, scale folded below
-                            } else if constexpr (BIAS == 1) {
-                                x = keep[e] ? s[i] * qk_scale : s[i] * qk_scale + kMask;
-                            } else {
-                                x = s[i] * p.sm_scale + bv[e];               // natural units
-                            }
-                            s[i] = x;
-                            mx = fmaxf(mx, x);
-                        }
+                for (int e = 0; e < 4; e++) {
+                    const int i = q4 * 4 + e;
+                    float x;
+                    if constexpr (MASKED) {
+                        x = __fmul_rn(s[i], qk_scale);
+                        const int n = n0 + nh + nl + e;
+                        float t = (n >= N) ? kMask : 0.f;
+                        if (CAUSAL) t += (my_m < n) ? kMask : 0.f;
+                        float add = 0.f;
+                        if (BIAS == 1) add = keep[e] ? 0.f : kMask;
+                        if (BIAS >= 2) add = __fmul_rn(bv[e], kLog2e);
+                        if (BIAS != 0) add = (n >= N) ? kMask : add;  // out-of-range bias reads as masked
+                        x = __fadd_rn(x, __fadd_rn(t, add));
+                    } else if constexpr (BIAS == 0) {
+                        x = s[i];                                    // raw score, scale folded below
+                    } else if constexpr (BIAS == 1) {
+                        x = keep[e] ? s[i] * qk_scale : s[i] * qk_scale + kMask;
+                    } else {
+                        x = s[i] * p.sm_scale + bv[e];               // natural units
                     }
+                    s[i] = x;
+                    mx = fmaxf(mx, x);
                 }
-                // units of x: log2 (MASKED, bool bias), raw dot product (no bias), natural (float bias)
-                constexpr bool RAW = !MASKED && BIAS == 0;
-                constexpr bool NAT = !MASKED && BIAS >= 2;
-                const float to_log2 = RAW ? qk_scale : (NAT ? kLog2e : 1.f);
-                mx = pair_max(mx) * to_log2;
-                const bool raise = mx > m_i + 8.f;
-                if (__builtin_amdgcn_ballot_w64(raise) != 0) {
-                    const float m_new = raise ? mx : m_i;
-                    const float alpha = fast_exp2(m_i - m_new);
-                    m_i = m_new;
-                    l_i *= alpha;
-#pragma unroll
-                    for (int db = 0; db < C::DB; db++)
-#pragma unroll
-                        for (int i = 0; i < 16; i++) o_acc[db][i] *= alpha;
-                }
-                float rs = 0.f;
-                {
-#pragma unroll
-                    for (int i = 0; i < 16; i++) {
-                        float pv;
-                        if constexpr (RAW || NAT) pv = fast_exp2(__builtin_fmaf(s[i], to_log2, -m_i));
-                        else pv = fast_exp2(s[i] - m_i);
-                        rs += pv;
-                        pb[i >> 3][i & 7] = (T)pv;
-                    }
-                }
-                l_i += rs;  // per-lane partial sum; the two halves are added at the end
-            };
-            if constexpr (TILE_MASKED) {
-                if (need_mask || !(qk_scale > 0.f)) softmax_step(std::true_type{});
-                else softmax_step(std::false_type{});
-            } else {
-                softmax_step(std::false_type{});
             }
+            // units of x: log2 (MASKED, bool bias), raw dot product (no bias), natural (float bias)
+            constexpr bool RAW = !MASKED && BIAS == 0;
+            constexpr bool NAT = !MASKED && BIAS >= 2;
+            const float to_log2 = RAW ? qk_scale : (NAT ? kLog2e : 1.f);
+            mx = pair_max(mx) * to_log2;
+            const bool raise = mx > m_i + 8.f;
+            if (__builtin_amdgcn_ballot_w64(raise) != 0) {
+                const float m_new = raise ? mx : m_i;
+                const float alpha = fast_exp2(m_i - m_new);
+                m_i = m_new;
+                l_i *= alpha;
+#pragma unroll
+                for (int db = 0; db < C::DB; db++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++) o_acc[db][i] *= alpha;
+            }
+            float rs = 0.f;
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                float pv;
+                if constexpr (RAW || NAT) pv = fast_exp2(__builtin_fmaf(s[i], to_log2, -m_i));
+                else pv = fast_exp2(s[i] - m_i);
+                rs += pv;
+                pb[i >> 3][i & 7] = (T)pv;
+            }
+            l_i += rs;  // per-lane partial sum; the two halves of a row are added at the end
+        };
+        if constexpr (STEP_MASKED) {
+            if (need_mask || !(qk_scale > 0.f)) softmax_step(std::true_type{});
+            else softmax_step(std::false_type{});
+        } else {
+            softmax_step(std::false_type{});
+        }
 
-            // ---- O^T += V^T P^T : A = V^T gathered down the columns of the V tile ----
+        // ---- O^T += V^T P^T : A = V^T gathered down the columns of the V rows ----
 #pragma unroll
-            for (int kk = 0; kk < 2; kk++) {
+        for (int kk = 0; kk < 2; kk++) {
 #pragma unroll
-                for (int db = 0; db < C::DB; db++) {
-                    T8 a = SW::template col8<T8>(v_lds, lane, nh + kk * 16, db * 32);
-                    o_acc[db] = mfma32(a, pb[kk], o_acc[db]);
-                }
+            for (int db = 0; db < C::DB; db++) {
+                T8 a = SW::template col8<T8>(v_lds, lane, nh + kk * 16, db * 32);
+                o_acc[db] = mfma32(a, pb[kk], o_acc[db]);
             }
+        }
         }
     };
 
-    int n_fast = N / BN;  // leading tiles that need no masks
-    if (CAUSAL) n_fast = n_fast < (m0 + 1) / BN ? n_fast : (m0 + 1) / BN;
-    if (n_fast > n_tiles) n_fast = n_tiles;
+    int n_fast = N / BK;  // leading steps that need no masks
+    if (CAUSAL) n_fast = n_fast < (m0 + 1) / BK ? n_fast : (m0 + 1) / BK;
+    if (n_fast > n_steps) n_fast = n_steps;
     if (!(qk_scale > 0.f)) n_fast = 0;
+
+    auto run = [&](auto bv_tag) {
+        constexpr bool BV = decltype(bv_tag)::value;
+        // prologue in the order the steps assume: the first bias slices, then K/V of a step followed
+        // by the bias slice issued in the same step
+        if constexpr (BV) {
+#pragma unroll
+            for (int i = 0; i < C::NBS - 1 - C::LA; i++) issue_bias(i);
+        }
+#pragma unroll
+        for (int i = 0; i < C::LA; i++) {
+            issue_kv(i);
+            if constexpr (BV) issue_bias(C::NBS - 1 - C::LA + i);
+        }
 #pragma unroll 1
-    for (int j = 0; j < n_fast; j++) tile_step(j, std::false_type{});
+        for (int k = 0; k < n_fast; k++) kv_step(k, std::false_type{}, bv_tag);
 #pragma unroll 1
-    for (int j = n_fast; j < n_tiles; j++) tile_step(j, std::true_type{});
+        for (int k = n_fast; k < n_steps; k++) kv_step(k, std::true_type{}, bv_tag);
+    };
+    if (BIAS != 0 && p.bias_vec) run(std::true_type{});
+    else run(std::false_type{});
 
     // ---- epilogue (flash_attention.py:188-194) ----
     const float l_tot = pair_sum(l_i);
     const float inv_l = 1.f / l_tot;
     if (g == 0 && my_m < M) p.lse[((int64_t)b * p.H + h) * M + my_m] = m_i + fast_log2(l_tot);
 
-    __syncthreads();  // K/V tiles are dead: reuse their LDS for the output tile
+    wait_vmcnt<0>();  // copies issued past the last step must not land in the output tile
+    __syncthreads();  // K/V slots are dead: reuse their LDS for the output tile
     T* o_lds = reinterpret_cast<T*>(smem) + wave * 32 * OS;
 #pragma unroll
     for (int db = 0; db < C::DB; db++) {

@@ -43,17 +43,19 @@ __global__ __launch_bounds__(256) void fa_bwd_prep_kernel(const BwdParams p) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// dQ kernel: a work-group owns 128 query rows (Q^T and dO^T in registers), streams K / V tiles
+// dQ kernel: a work-group owns 128 query rows (Q^T and dO^T in registers), streams K / V rows
 // and recomputes S^T = K Q^T and dP^T = V dO^T, so that dS^T sits in the accumulator layout that
-// dQ^T += K^T dS^T wants as its B operand.  Replaces _attn_bwd_dq (flash_attention.py:458-646).
+// dQ^T += K^T dS^T wants as its B operand.  K, V and the bias slices arrive through the same
+// counted direct-to-LDS copy rings as in the forward kernel.  Replaces _attn_bwd_dq
+// (flash_attention.py:458-646).
 template <typename T, int D, int BIAS, bool CAUSAL>
-__global__ __launch_bounds__(256, (RowCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_dq_kernel(const BwdParams p) {
-    typedef RowCfg<D, BIAS> C;
+__global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_dq_kernel(const BwdParams p) {
+    typedef StreamCfg<D, BIAS> C;
     typedef Swz<D> SW;
     typedef typename VecOf<T>::v8 T8;
     typedef typename VecOf<T>::v4 T4;
     typedef typename BiasElem<BIAS>::type E;
-    constexpr int BM = C::BM, BN = C::BN, OS = C::OS, CPR = C::CPR;
+    constexpr int BM = C::BM, BK = C::BK, OS = C::OS, CPR = C::CPR;
 
     __shared__ __align__(16) unsigned char smem[C::LDS_BYTES];
 
@@ -71,14 +73,10 @@ __global__ __launch_bounds__(256, (RowCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_dq_
     const int my_m = mw + r;
 
     const T* qp = reinterpret_cast<const T*>(p.q) + (int64_t)b * p.sq.b + (int64_t)h * p.sq.h;
-    const char* kbase = reinterpret_cast<const char*>(reinterpret_cast<const T*>(p.k) + (int64_t)b * p.sk.b + (int64_t)h * p.sk.h);
-    const char* vbase = reinterpret_cast<const char*>(reinterpret_cast<const T*>(p.v) + (int64_t)b * p.sv.b + (int64_t)h * p.sv.h);
+    const T* kp = reinterpret_cast<const T*>(p.k) + (int64_t)b * p.sk.b + (int64_t)h * p.sk.h;
+    const T* vp = reinterpret_cast<const T*>(p.v) + (int64_t)b * p.sv.b + (int64_t)h * p.sv.h;
     const E* bp = nullptr;
-    unsigned char* bias_lds = nullptr;
-    if (BIAS != 0) {
-        bp = reinterpret_cast<const E*>(p.bias) + (int64_t)b * p.sbias.b + (int64_t)h * p.sbias.h;
-        bias_lds = smem + C::KV_BYTES + wave * 32 * C::BROW;
-    }
+    if (BIAS != 0) bp = reinterpret_cast<const E*>(p.bias) + (int64_t)b * p.sbias.b + (int64_t)h * p.sbias.h;
 
     // Q^T and dO^T as B operands: column my_m, k = d
     const T* dop = reinterpret_cast<const T*>(p.dout) + (int64_t)b * p.sdo.b + (int64_t)h * p.sdo.h;
@@ -100,10 +98,10 @@ __global__ __launch_bounds__(256, (RowCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_dq_
         delta_i = p.delta[((int64_t)b * p.H + h) * M + my_m];
     }
 
-    int n_tiles = (N + BN - 1) / BN;
+    int n_steps = (N + BK - 1) / BK;
     if (CAUSAL) {
-        int last = (m0 + BM - 1) / BN + 1;  // tiles holding keys <= last row of this work-group
-        n_tiles = n_tiles < last ? n_tiles : last;
+        int last = (m0 + BM - 1) / BK + 1;  // steps holding keys <= last row of this work-group
+        n_steps = n_steps < last ? n_steps : last;
     }
 
     const float qk_scale = p.sm_scale * kLog2e;
@@ -113,118 +111,29 @@ __global__ __launch_bounds__(256, (RowCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_dq_
 #pragma unroll
         for (int i = 0; i < 16; i++) dq_acc[db][i] = 0.f;
 
-    // ---- K / V tiles: global -> LDS without passing through registers.  Chunk c of a tile
-    // (row c / CPR, LDS chunk c % CPR) is copied by thread c % 256 in copy c / 256; the LDS chunk
-    // holds global chunk (c % CPR) ^ f(row), which is the swizzle the readers expect.
-    unsigned koff[C::NCH], voff[C::NCH];  // byte offsets of this lane's source chunks in a full tile
-#pragma unroll
-    for (int it = 0; it < C::NCH; it++) {
-        const int c = it * C::NT + tid;
-        const int row = c / CPR, src = (c % CPR) ^ SW::f(row);
-        koff[it] = (unsigned)(row * (int)p.sk.s * 2 + src * 16);
-        voff[it] = (unsigned)(row * (int)p.sv.s * 2 + src * 16);
-    }
-    auto issue_tile = [&](int j, int buf) {
-        const int n0 = j * BN;
-        const char* kt = kbase + (int64_t)n0 * p.sk.s * 2;
-        const char* vt = vbase + (int64_t)n0 * p.sv.s * 2;
-        unsigned char* k_dst = smem + buf * C::TILE_BYTES;
-        unsigned char* v_dst = smem + (2 + buf) * C::TILE_BYTES;
-        const bool full = n0 + BN <= N;
-#pragma unroll
-        for (int it = 0; it < C::NCH; it++) {
-            const int c0 = it * C::NT + wave * 64;  // first chunk of this wave's copy
-            if (c0 < C::TILE_CHUNKS) {
-                unsigned ko = koff[it], vo = voff[it];
-                if (!full) {  // rows past the last key re-read the last key; the scores are masked
-                    const int c = c0 + lane;
-                    int row = c / CPR;
-                    const int src = (c % CPR) ^ SW::f(row);
-                    row = row < N - n0 ? row : N - n0 - 1;
-                    ko = (unsigned)(row * (int)p.sk.s * 2 + src * 16);
-                    vo = (unsigned)(row * (int)p.sv.s * 2 + src * 16);
-                }
-                g2lds16(kt + ko, k_dst + c0 * 16);
-                g2lds16(vt + vo, v_dst + c0 * 16);
-            }
-        }
-    };
+    KeyStream<T, D, BIAS> ks_;
+    ks_.init(smem, kp, vp, bp, p.sk.s, p.sv.s, p.sbias.m, p.sbias.n, M, N, mw, wave, lane);
 
-    // ---- bias tile of this wave (32 rows x 64 keys): global -> registers one tile ahead ----
-    i32x4 breg[C::BCH > 0 ? C::BCH : 1];
-    int boff[C::BCH > 0 ? C::BCH : 1];
-    __amdgpu_buffer_rsrc_t brsrc = make_buffer(nullptr, 0);
-    if constexpr (BIAS != 0) {
-        constexpr int CH_ROW = 4 * C::ES;  // 16-byte chunks per 64-key row
+    // One step of the K/V stream.  Interior steps (every key in range and visible to every row of
+    // the work-group) run with STEP_MASKED = false: no range checks, no mask arithmetic.  BV: the
+    // bias slices come by copy (rows that allow aligned 16-byte chunks), else element by element.
+    auto kv_step = [&](int k, auto step_tag, auto bv_tag) {
+        constexpr bool STEP_MASKED = decltype(step_tag)::value;
+        constexpr bool BV = decltype(bv_tag)::value;
+        const int n0 = k * BK;
+        ks_.template begin_step<BV>(k);
+        const T* k_lds = ks_.k_lds(k);
+        const T* v_lds = ks_.v_lds(k);
+        const unsigned char* b_lds = ks_.b_lds(k);
+        static_assert(BIAS == 0 || C::NH == 1, "a bias slot covers one 32-key block");
+        // The step is consumed 32 keys at a time, so that only one 32 x 32 score block is live.
 #pragma unroll
-        for (int it = 0; it < C::BCH; it++) {
-            const int c = it * 64 + lane;
-            boff[it] = (c / CH_ROW) * (int)p.sbias.m * C::ES + (c % CH_ROW) * 16;
-        }
-        // everything from the first row of this wave to the end of the (b, h) slice
-        brsrc = make_buffer(bp + (int64_t)mw * p.sbias.m, ((int64_t)(M - 1 - mw) * p.sbias.m + N) * C::ES);
-    }
-    auto prefetch_bias = [&](int j) {
-        if constexpr (BIAS != 0) {
-            if (p.bias_vec) {
-#pragma unroll
-                for (int it = 0; it < C::BCH; it++) breg[it] = buf_load16(brsrc, boff[it], j * BN * C::ES);
-            }
-        }
-    };
-
-    if (n_tiles > 0) {
-        issue_tile(0, 0);
-        prefetch_bias(0);
-    }
-
-    // One tile of the K/V stream.  Interior tiles (every key in range and visible to every row of
-    // the work-group) run with TILE_MASKED = false: no range checks, no mask arithmetic.
-    auto tile_step = [&](int j, auto tile_tag) {
-        constexpr bool TILE_MASKED = decltype(tile_tag)::value;
-        const int n0 = j * BN;
-        const int buf = j & 1;
-        const T* k_lds = reinterpret_cast<const T*>(smem + buf * C::TILE_BYTES);
-        const T* v_lds = reinterpret_cast<const T*>(smem + (2 + buf) * C::TILE_BYTES);
-        __builtin_amdgcn_s_waitcnt(0);  // this thread's copies of tile j (and its bias chunks) have landed
-        if constexpr (BIAS != 0) {
-            if (p.bias_vec) {
-#pragma unroll
-                for (int it = 0; it < C::BCH; it++) {
-                    constexpr int CH_ROW = 4 * C::ES;
-                    const int c = it * 64 + lane;
-                    const int row = c / CH_ROW;
-                    lds_write16(bias_lds + row * C::BROW + (((c % CH_ROW) ^ C::bswz(row)) << 4), breg[it]);
-                }
-            } else {
-                // unaligned bias rows or non-unit key stride: one element per lane per row
-#pragma unroll 1
-                for (int row = 0; row < 32; row++) {
-                    int n = n0 + lane;
-                    E val = (E)0.f;
-                    if (mw + row < M && n < N)
-                        val = bp[(int64_t)(mw + row) * p.sbias.m + (int64_t)n * p.sbias.n];
-                    const int byte = lane * C::ES;
-                    *reinterpret_cast<E*>(bias_lds + row * C::BROW + (((byte >> 4) ^ C::bswz(row)) << 4) + (byte & 15)) = val;
-                }
-            }
-        }
-        __syncthreads();  // tile j is complete in LDS; nobody still reads the buffer of tile j - 1
-        if (j + 1 < n_tiles) {
-            issue_tile(j + 1, buf ^ 1);
-            prefetch_bias(j + 1);
-        }
-
-        // The 64-key tile is consumed as two 32-key halves, each with its own softmax step, so
-        // that only one 32 x 32 score block is live at a time.
-#pragma unroll
-        for (int nb = 0; nb < 2; nb++) {
-            const int nh = nb * 32;  // first key of this half inside the tile
-            __builtin_amdgcn_sched_barrier(0);  // keep the halves apart: one score block live at a time
-            // halves entirely above this wave's diagonal contribute nothing
-            if (TILE_MASKED && CAUSAL && n0 + nh > mw + 31) continue;
-            if (TILE_MASKED && n0 + nh >= N) continue;
-            const bool need_mask = TILE_MASKED && ((n0 + nh + 32 > N) || (CAUSAL && n0 + nh + 31 > mw));
+        for (int nb = 0; nb < C::NH; nb++) {
+            const int nh = nb * 32;  // first key of this block inside the step
+            __builtin_amdgcn_sched_barrier(0);  // keep the blocks apart
+            // blocks entirely above this wave's diagonal or past the last key contribute nothing
+            if (STEP_MASKED && ((CAUSAL && n0 + nh > mw + 31) || n0 + nh >= N)) continue;
+            const bool need_mask = STEP_MASKED && ((n0 + nh + 32 > N) || (CAUSAL && n0 + nh + 31 > mw));
 
             // ---- S^T = K Q^T : s[i] is key n0 + nh + 8 (i/4) + 4 g + i%4, query my_m ----
             f32x16 s;
@@ -253,20 +162,20 @@ __global__ __launch_bounds__(256, (RowCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_dq_
                 constexpr bool MASKED = decltype(masked_tag)::value;
 #pragma unroll
                 for (int q4 = 0; q4 < 4; q4++) {
-                    const int nl = nh + 8 * q4 + 4 * g;  // first of 4 consecutive keys
+                    const int nl = 8 * q4 + 4 * g;  // first of 4 consecutive keys of the block
                     float bv[4] = {0.f, 0.f, 0.f, 0.f};  // bias in natural units
                     bool keep[4] = {true, true, true, true};
                     if constexpr (BIAS == 1) {
-                        unsigned int w = *reinterpret_cast<const unsigned int*>(bias_lds + r * C::BROW + (((nl >> 4) ^ C::bswz(r)) << 4) + (nl & 15));
+                        unsigned int w = *reinterpret_cast<const unsigned int*>(b_lds + ks_.b_off(r, nl));
 #pragma unroll
                         for (int e = 0; e < 4; e++) keep[e] = ((w >> (8 * e)) & 0xffu) != 0;
                     } else if constexpr (BIAS == 2 || BIAS == 3) {
                         typedef typename VecOf<E>::v4 B4;
-                        B4 hv = *reinterpret_cast<const B4*>(bias_lds + r * C::BROW + (((nl >> 3) ^ C::bswz(r)) << 4) + ((nl * 2) & 15));
+                        B4 hv = *reinterpret_cast<const B4*>(b_lds + ks_.b_off(r, nl));
 #pragma unroll
                         for (int e = 0; e < 4; e++) bv[e] = (float)hv[e];
                     } else if constexpr (BIAS == 4) {
-                        f32x4 w = *reinterpret_cast<const f32x4*>(bias_lds + r * C::BROW + (((nl >> 2) ^ C::bswz(r)) << 4));
+                        f32x4 w = *reinterpret_cast<const f32x4*>(b_lds + ks_.b_off(r, nl));
 #pragma unroll
                         for (int e = 0; e < 4; e++) bv[e] = w[e];
                     }
@@ -276,7 +185,7 @@ __global__ __launch_bounds__(256, (RowCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_dq_
                         float pv;
                         if constexpr (MASKED) {
                             float x = __fmul_rn(s[i], qk_scale);
-                            const int n = n0 + nl + e;
+                            const int n = n0 + nh + nl + e;
                             const bool oob = (n >= N) || (my_m >= M);
                             float t = oob ? kMask : 0.f;
                             if (CAUSAL) t += (my_m < n) ? kMask : 0.f;
@@ -297,7 +206,7 @@ __global__ __launch_bounds__(256, (RowCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_dq_
                     }
                 }
             };
-            if constexpr (TILE_MASKED) {
+            if constexpr (STEP_MASKED) {
                 if (need_mask || m0 + BM > M) ds_step(std::true_type{});
                 else ds_step(std::false_type{});
             } else {
@@ -316,17 +225,23 @@ __global__ __launch_bounds__(256, (RowCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_dq_
         }
     };
 
-    int n_fast = N / BN;  // leading tiles that need no masks
-    if (CAUSAL) n_fast = n_fast < (m0 + 1) / BN ? n_fast : (m0 + 1) / BN;
-    if (n_fast > n_tiles) n_fast = n_tiles;
+    int n_fast = N / BK;  // leading steps that need no masks
+    if (CAUSAL) n_fast = n_fast < (m0 + 1) / BK ? n_fast : (m0 + 1) / BK;
+    if (n_fast > n_steps) n_fast = n_steps;
     if (!(qk_scale > 0.f) || m0 + BM > M) n_fast = 0;
+    auto run = [&](auto bv_tag) {
+        constexpr bool BV = decltype(bv_tag)::value;
+        ks_.template prologue<BV>();
 #pragma unroll 1
-    for (int j = 0; j < n_fast; j++) tile_step(j, std::false_type{});
+        for (int k = 0; k < n_fast; k++) kv_step(k, std::false_type{}, bv_tag);
 #pragma unroll 1
-    for (int j = n_fast; j < n_tiles; j++) tile_step(j, std::true_type{});
+        for (int k = n_fast; k < n_steps; k++) kv_step(k, std::true_type{}, bv_tag);
+    };
+    if (BIAS != 0 && p.bias_vec) run(std::true_type{});
+    else run(std::false_type{});
 
     // ---- epilogue: dq = dQ * sm_scale (flash_attention.py:644-646) ----
-    __syncthreads();  // K/V tiles are dead: reuse their LDS for the output tile
+    ks_.drain();  // K/V slots are dead and no copy is in flight: reuse their LDS for the output tile
     T* o_lds = reinterpret_cast<T*>(smem) + wave * 32 * OS;
 #pragma unroll
     for (int db = 0; db < C::DB; db++) {

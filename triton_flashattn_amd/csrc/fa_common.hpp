@@ -228,34 +228,7 @@ template <> struct BiasElem<2> { typedef _Float16 type; };
 template <> struct BiasElem<3> { typedef __bf16 type; };
 template <> struct BiasElem<4> { typedef float type; };
 
-// Tiling of the kernels in which a work-group owns 128 query rows (4 waves x 32 rows) and
-// streams keys in tiles of 64 through double-buffered LDS: the forward and the dQ kernel.
-template <int D, int BIAS> struct RowCfg {
-    static constexpr int BM = 128, BN = 64, NT = 256;
-    static constexpr int DP = D < 32 ? 32 : D;       // head dim padded to one 32-wide MFMA block
-    static constexpr int OS = DP + 8;                // O staging row stride (elements)
-    static constexpr int CPR = D / 8;                // 16-byte chunks per row
-    static constexpr int TILE_CHUNKS = BN * CPR;     // 16-byte chunks per K (or V) tile
-    static constexpr int NCH = (TILE_CHUNKS + NT - 1) / NT;  // direct-to-LDS copies per thread per tile
-    static constexpr int KSTEPS = D / 16;            // MFMA k-steps of Q K^T
-    static constexpr int DB = DP / 32;               // 32-wide blocks of the head dim
-    static constexpr int ES = BIAS == 0 ? 0 : (BIAS == 1 ? 1 : (BIAS == 4 ? 4 : 2));
-    static constexpr int BROW = 64 * ES;             // bias tile row: 64 keys, unpadded, chunk-swizzled
-    // 16-byte chunk c of bias row `row` is stored at chunk c ^ bswz(row)
-    __device__ static __forceinline__ int bswz(int row) {
-        return ES == 4 ? (row & 15) : (ES == 2 ? (row & 7) : ((row >> 2) & 3));
-    }
-    static constexpr int BCH = 2 * ES;               // 16-byte bias chunks per lane per tile
-    static constexpr int TILE_BYTES = BN * D * 2;    // unpadded, swizzled
-    static constexpr int O_BYTES = BM * OS * 2;
-    static constexpr int KV_BYTES = 4 * TILE_BYTES > O_BYTES ? 4 * TILE_BYTES : O_BYTES;  // K[2], V[2]
-    static constexpr int BIAS_BYTES = 4 * 32 * BROW;
-    static constexpr int LDS_BYTES = KV_BYTES + BIAS_BYTES;
-    // two work-groups per CU whenever registers allow it
-    static constexpr int MIN_BLOCKS = D <= 128 ? 2 : 1;
-};
-
-// Tiling of the forward kernel: a work-group owns 128 query rows (4 waves x 32 rows) and streams
+// Tiling of the forward and the dQ kernel: a work-group owns 128 query rows (4 waves x 32 rows) and streams
 // keys in steps of NH blocks of 32.  K and V rows of a step and the bias slice of each wave reach
 // LDS through direct global -> LDS copies issued ahead of their use.  With a bias: steps of 32
 // keys, K/V in a ring of 3 slots (two steps ahead), the bias in a ring of 4 slots per wave (three
@@ -292,6 +265,137 @@ template <int D, int BIAS> struct StreamCfg {
     }
     // two work-groups per CU whenever registers and LDS allow it
     static constexpr int MIN_BLOCKS = (D <= 128 && LDS_BYTES <= 81920) ? 2 : 1;
+};
+
+// The copy machinery of the kernels tiled by StreamCfg (forward, dQ): one object per thread.
+// Completion of the copies is counted by hand: they complete in issue order and every wave issues
+// the same number every step, also past the last step (clamped rows, never used).
+template <typename T, int D, int BIAS> struct KeyStream {
+    typedef StreamCfg<D, BIAS> C;
+    typedef Swz<D> SW;
+    typedef typename BiasElem<BIAS>::type E;
+    unsigned char* smem;      // K slots, then V slots, then the bias rings of the four waves
+    unsigned char* bias_lds;  // this wave's ring of bias slots
+    const T* kp;
+    const T* vp;
+    const E* bp;              // (batch, head) slices
+    int64_t sk, sv, sbm, sbn; // row strides of K and V, row and key stride of the bias (elements)
+    int M, N, mw, lane;
+    unsigned k_off[C::KD], v_off[C::KD];
+    int c_idx[C::KD];
+
+    // K / V rows of a step: NKD copies of 1 KB each; copy ci fills bytes [1024 ci, 1024 ci + 1024) of
+    // the swizzled slot, so lane l of it fetches the chunk that lives at slot position 64 ci + l
+    // (row c / CPR, LDS chunk c % CPR holds global chunk (c % CPR) ^ f(row)).  Each wave issues KD
+    // of them (more than once where a step has fewer than four).
+    __device__ __forceinline__ void init(unsigned char* smem_, const T* kp_, const T* vp_, const E* bp_, int64_t sk_,
+                                         int64_t sv_, int64_t sbm_, int64_t sbn_, int M_, int N_, int mw_, int wave, int lane_) {
+        smem = smem_; kp = kp_; vp = vp_; bp = bp_; sk = sk_; sv = sv_; sbm = sbm_; sbn = sbn_;
+        M = M_; N = N_; mw = mw_; lane = lane_;
+        bias_lds = smem + C::KV_BYTES + wave * C::NBS * C::BSLOT;
+#pragma unroll
+        for (int i = 0; i < C::KD; i++) {
+            c_idx[i] = (wave * C::KD + i) % C::NKD;
+            const int c = c_idx[i] * 64 + lane;
+            const int row = c / C::CPR, src = (c % C::CPR) ^ SW::f(row);
+            k_off[i] = (unsigned)(row * (int)sk * 2 + src * 16);
+            v_off[i] = (unsigned)(row * (int)sv * 2 + src * 16);
+        }
+    }
+    __device__ __forceinline__ const T* k_lds(int k) const { return reinterpret_cast<const T*>(smem + (k % C::NKV) * C::STEP_BYTES); }
+    __device__ __forceinline__ const T* v_lds(int k) const { return reinterpret_cast<const T*>(smem + (C::NKV + k % C::NKV) * C::STEP_BYTES); }
+    __device__ __forceinline__ unsigned char* b_lds(int k) const { return bias_lds + (k % C::NBS) * C::BSLOT; }
+    // byte offset of bias (row, key .. key + 3) inside a slot
+    __device__ static __forceinline__ int b_off(int row, int key) {
+        const int byte = key * C::ES;
+        return row * C::BROW + (((byte >> 4) ^ C::bswz(row)) << 4) + (byte & 15);
+    }
+
+    // Rows past N re-read row N - 1 (their scores are masked); a step past the end is that row
+    // over and over, so that offsets never go negative.
+    __device__ __forceinline__ void issue_kv(int k) {
+        const int n0 = k * C::BK < N ? k * C::BK : N - 1;
+        const T* kt = kp + (int64_t)n0 * sk;
+        const T* vt = vp + (int64_t)n0 * sv;
+        unsigned char* k_dst = smem + (k % C::NKV) * C::STEP_BYTES;
+        unsigned char* v_dst = smem + (C::NKV + k % C::NKV) * C::STEP_BYTES;
+        const bool full = n0 + C::BK <= N;
+#pragma unroll
+        for (int i = 0; i < C::KD; i++) {
+            unsigned ko = k_off[i], vo = v_off[i];
+            if (!full) {
+                const int c = c_idx[i] * 64 + lane;
+                int row = c / C::CPR;
+                const int src = (c % C::CPR) ^ SW::f(row);
+                row = row < N - n0 ? row : N - 1 - n0;
+                ko = (unsigned)(row * (int)sk * 2 + src * 16);
+                vo = (unsigned)(row * (int)sv * 2 + src * 16);
+            }
+            g2lds16_untracked(kt, ko, k_dst + c_idx[i] * 1024);
+            g2lds16_untracked(vt, vo, v_dst + c_idx[i] * 1024);
+        }
+    }
+    // Bias slice of this wave for step k (32 rows x 32 keys) -> ring slot k % NBS.  Position c =
+    // 64 it + lane of the slot (row c / BCPR, LDS chunk c % BCPR) holds chunk (c % BCPR) ^ bswz(row)
+    // of the row.  Rows past M re-read row M - 1 (never stored) and chunks that start past N
+    // re-read column 0 (masked).
+    __device__ __forceinline__ void issue_bias(int k) {
+        if constexpr (BIAS != 0) {
+            unsigned char* dst = b_lds(k);
+#pragma unroll
+            for (int it = 0; it < C::BCH; it++) {
+                const int c = it * 64 + lane;
+                const int row = c / C::BCPR;
+                int m = mw + row;
+                int n = k * C::BK + ((c % C::BCPR) ^ C::bswz(row)) * C::EPC;
+                m = m < M ? m : M - 1;
+                n = n < N ? n : 0;
+                g2lds16_untracked(bp + (int64_t)m * sbm + n, dst + it * 1024);
+            }
+        }
+    }
+    // Before the first step, in the order the steps assume: the first bias slices, then K/V of a
+    // step followed by the bias slice issued in the same step.  BV: the bias slices come by copy.
+    template <bool BV> __device__ __forceinline__ void prologue() {
+        if constexpr (BV) {
+#pragma unroll
+            for (int i = 0; i < C::NBS - 1 - C::LA; i++) issue_bias(i);
+        }
+#pragma unroll
+        for (int i = 0; i < C::LA; i++) {
+            issue_kv(i);
+            if constexpr (BV) issue_bias(C::NBS - 1 - C::LA + i);
+        }
+    }
+    // Top of step k: wait for its K/V rows (and with them its bias slice, issued earlier), publish
+    // them, and issue the copies that go into the slots step k - 1 has just left.
+    template <bool BV> __device__ __forceinline__ void begin_step(int k) {
+        static_assert(BIAS == 0 || C::LA < C::NBS - 1, "the bias slice of a step must be issued before its K/V rows");
+        constexpr int OPS = 2 * C::KD + (BV ? C::BCH : 0);  // copies per wave per step
+        // K/V of this step were issued LA steps ago; the bias copies issued right after them and
+        // the copies of the steps since may still be in flight
+        wait_vmcnt<(BV ? C::BCH : 0) + OPS*(C::LA - 1)>();
+        lds_barrier();
+        issue_kv(k + C::LA);
+        if constexpr (BV) issue_bias(k + C::NBS - 1);
+        if constexpr (BIAS != 0 && !BV) {
+            // unaligned bias rows or non-unit key stride: one element per lane per row
+            if (lane < 32) {
+#pragma unroll 1
+                for (int row = 0; row < 32; row++) {
+                    const int n = k * C::BK + lane;
+                    E val = (E)0.f;
+                    if (mw + row < M && n < N) val = bp[(int64_t)(mw + row) * sbm + (int64_t)n * sbn];
+                    *reinterpret_cast<E*>(b_lds(k) + b_off(row, lane)) = val;
+                }
+            }
+        }
+    }
+    // After the last step: nothing may land in LDS that is about to be reused.
+    __device__ __forceinline__ void drain() {
+        wait_vmcnt<0>();
+        __syncthreads();
+    }
 };
 
 // Work-group id -> (tile, batch*head).  Work-groups are dealt round-robin to the 8 XCDs; when

@@ -54,11 +54,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_
     const T* kp = reinterpret_cast<const T*>(p.k) + (int64_t)b * p.sk.b + (int64_t)h * p.sk.h;
     const T* vp = reinterpret_cast<const T*>(p.v) + (int64_t)b * p.sv.b + (int64_t)h * p.sv.h;
     const E* bp = nullptr;
-    unsigned char* bias_lds = nullptr;  // this wave's ring of bias slots
-    if (BIAS != 0) {
-        bp = reinterpret_cast<const E*>(p.bias) + (int64_t)b * p.sbias.b + (int64_t)h * p.sbias.h;
-        bias_lds = smem + C::KV_BYTES + wave * C::NBS * C::BSLOT;
-    }
+    if (BIAS != 0) bp = reinterpret_cast<const E*>(p.bias) + (int64_t)b * p.sbias.b + (int64_t)h * p.sbias.h;
 
     // Q^T as B operand: column my_m, k = d
     T8 qreg[C::KSTEPS];
@@ -83,62 +79,8 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_
 #pragma unroll
         for (int i = 0; i < 16; i++) o_acc[db][i] = 0.f;
 
-    // ---- K / V rows of a step: NKD copies of 1 KB each; copy ci fills bytes [1024 ci, 1024 ci + 1024)
-    // of the swizzled slot, so lane l of it fetches the chunk that lives at slot position 64 ci + l
-    // (row c / CPR, LDS chunk c % CPR holds global chunk (c % CPR) ^ f(row)).  Each wave issues KD
-    // of them (more than once where a step has fewer than four).  Rows past N re-read row N - 1:
-    // their scores are masked.
-    unsigned k_off[C::KD], v_off[C::KD];
-    int c_idx[C::KD];
-#pragma unroll
-    for (int i = 0; i < C::KD; i++) {
-        c_idx[i] = (wave * C::KD + i) % C::NKD;
-        const int c = c_idx[i] * 64 + lane;
-        const int row = c / CPR, src = (c % CPR) ^ SW::f(row);
-        k_off[i] = (unsigned)(row * (int)p.sk.s * 2 + src * 16);
-        v_off[i] = (unsigned)(row * (int)p.sv.s * 2 + src * 16);
-    }
-    auto issue_kv = [&](int k) {
-        const int n0 = k * BK < N ? k * BK : N - 1;  // a step past the end is the last row over and over
-        const T* kt = kp + (int64_t)n0 * p.sk.s;
-        const T* vt = vp + (int64_t)n0 * p.sv.s;
-        unsigned char* k_dst = smem + (k % C::NKV) * C::STEP_BYTES;
-        unsigned char* v_dst = smem + (C::NKV + k % C::NKV) * C::STEP_BYTES;
-        const bool full = n0 + BK <= N;
-#pragma unroll
-        for (int i = 0; i < C::KD; i++) {
-            unsigned ko = k_off[i], vo = v_off[i];
-            if (!full) {
-                const int c = c_idx[i] * 64 + lane;
-                int row = c / CPR;
-                const int src = (c % CPR) ^ SW::f(row);
-                row = row < N - n0 ? row : N - 1 - n0;
-                ko = (unsigned)(row * (int)p.sk.s * 2 + src * 16);
-                vo = (unsigned)(row * (int)p.sv.s * 2 + src * 16);
-            }
-            g2lds16_untracked(kt, ko, k_dst + c_idx[i] * 1024);
-            g2lds16_untracked(vt, vo, v_dst + c_idx[i] * 1024);
-        }
-    };
-    // ---- bias slice of this wave for step k (32 rows x 32 keys) -> ring slot k % NBS.  Position c =
-    // 64 it + lane of the slot (row c / BCPR, LDS chunk c % BCPR) holds chunk (c % BCPR) ^ bswz(row)
-    // of the row.  Rows past M re-read row M - 1 (never stored) and chunks that start past N
-    // re-read column 0 (masked).
-    auto issue_bias = [&](int k) {
-        if constexpr (BIAS != 0) {
-            unsigned char* dst = bias_lds + (k % C::NBS) * C::BSLOT;
-#pragma unroll
-            for (int it = 0; it < C::BCH; it++) {
-                const int c = it * 64 + lane;
-                const int row = c / C::BCPR;
-                int m = mw + row;
-                int n = k * BK + ((c % C::BCPR) ^ C::bswz(row)) * C::EPC;
-                m = m < M ? m : M - 1;
-                n = n < N ? n : 0;
-                g2lds16_untracked(bp + (int64_t)m * p.sbias.m + n, dst + it * 1024);
-            }
-        }
-    };
+    KeyStream<T, D, BIAS> ks_;
+    ks_.init(smem, kp, vp, bp, p.sk.s, p.sv.s, p.sbias.m, p.sbias.n, M, N, mw, wave, lane);
 
     // One step of the K/V stream.  Interior steps (every key in range and visible to every row of
     // the work-group) run with STEP_MASKED = false: no range checks, no mask arithmetic.  BV: the
@@ -146,30 +88,11 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_
     auto kv_step = [&](int k, auto step_tag, auto bv_tag) {
         constexpr bool STEP_MASKED = decltype(step_tag)::value;
         constexpr bool BV = decltype(bv_tag)::value;
-        constexpr int OPS = 2 * C::KD + (BV ? C::BCH : 0);  // copies per wave per step
         const int n0 = k * BK;
-        const T* k_lds = reinterpret_cast<const T*>(smem + (k % C::NKV) * C::STEP_BYTES);
-        const T* v_lds = reinterpret_cast<const T*>(smem + (C::NKV + k % C::NKV) * C::STEP_BYTES);
-        const unsigned char* b_lds = bias_lds + (k % C::NBS) * C::BSLOT;
-        // K/V of this step were issued LA steps ago; the bias copies issued right after them and
-        // the copies of the steps since may still be in flight
-        wait_vmcnt<(BV ? C::BCH : 0) + OPS*(C::LA - 1)>();
-        lds_barrier();  // step k is complete in LDS; nobody still reads the slot of step k - 1
-        issue_kv(k + C::LA);
-        if constexpr (BV) issue_bias(k + C::NBS - 1);
-        if constexpr (BIAS != 0 && !BV) {
-            // unaligned bias rows or non-unit key stride: one element per lane per row
-            if (lane < 32) {
-#pragma unroll 1
-                for (int row = 0; row < 32; row++) {
-                    const int n = n0 + lane;
-                    E val = (E)0.f;
-                    if (mw + row < M && n < N) val = bp[(int64_t)(mw + row) * p.sbias.m + (int64_t)n * p.sbias.n];
-                    const int byte = lane * C::ES;
-                    *reinterpret_cast<E*>(bias_lds + (k % C::NBS) * C::BSLOT + row * C::BROW + (((byte >> 4) ^ C::bswz(row)) << 4) + (byte & 15)) = val;
-                }
-            }
-        }
+        ks_.template begin_step<BV>(k);
+        const T* k_lds = ks_.k_lds(k);
+        const T* v_lds = ks_.v_lds(k);
+        const unsigned char* b_lds = ks_.b_lds(k);
         static_assert(BIAS == 0 || C::NH == 1, "a bias slot covers one 32-key block");
         // The step is consumed 32 keys at a time, each block with its own softmax step, so that only
         // one 32 x 32 score block is live at a time.
@@ -205,20 +128,19 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_
 #pragma unroll
             for (int q4 = 0; q4 < 4; q4++) {
                 const int nl = 8 * q4 + 4 * g;            // first of 4 consecutive keys
-                const int byte = nl * C::ES;              // where they start in the bias row
                 float bv[4] = {0.f, 0.f, 0.f, 0.f};       // bias in natural units
                 bool keep[4] = {true, true, true, true};
                 if constexpr (BIAS == 1) {
-                    unsigned int w = *reinterpret_cast<const unsigned int*>(b_lds + r * C::BROW + (((byte >> 4) ^ C::bswz(r)) << 4) + (byte & 15));
+                    unsigned int w = *reinterpret_cast<const unsigned int*>(b_lds + ks_.b_off(r, nl));
 #pragma unroll
                     for (int e = 0; e < 4; e++) keep[e] = ((w >> (8 * e)) & 0xffu) != 0;
                 } else if constexpr (BIAS == 2 || BIAS == 3) {
                     typedef typename VecOf<E>::v4 B4;
-                    B4 hv = *reinterpret_cast<const B4*>(b_lds + r * C::BROW + (((byte >> 4) ^ C::bswz(r)) << 4) + (byte & 15));
+                    B4 hv = *reinterpret_cast<const B4*>(b_lds + ks_.b_off(r, nl));
 #pragma unroll
                     for (int e = 0; e < 4; e++) bv[e] = (float)hv[e];
                 } else if constexpr (BIAS == 4) {
-                    f32x4 w = *reinterpret_cast<const f32x4*>(b_lds + r * C::BROW + (((byte >> 4) ^ C::bswz(r)) << 4));
+                    f32x4 w = *reinterpret_cast<const f32x4*>(b_lds + ks_.b_off(r, nl));
 #pragma unroll
                     for (int e = 0; e < 4; e++) bv[e] = w[e];
                 }
@@ -300,17 +222,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_
 
     auto run = [&](auto bv_tag) {
         constexpr bool BV = decltype(bv_tag)::value;
-        // prologue in the order the steps assume: the first bias slices, then K/V of a step followed
-        // by the bias slice issued in the same step
-        if constexpr (BV) {
-#pragma unroll
-            for (int i = 0; i < C::NBS - 1 - C::LA; i++) issue_bias(i);
-        }
-#pragma unroll
-        for (int i = 0; i < C::LA; i++) {
-            issue_kv(i);
-            if constexpr (BV) issue_bias(C::NBS - 1 - C::LA + i);
-        }
+        ks_.template prologue<BV>();
 #pragma unroll 1
         for (int k = 0; k < n_fast; k++) kv_step(k, std::false_type{}, bv_tag);
 #pragma unroll 1
@@ -324,8 +236,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_
     const float inv_l = 1.f / l_tot;
     if (g == 0 && my_m < M) p.lse[((int64_t)b * p.H + h) * M + my_m] = m_i + fast_log2(l_tot);
 
-    wait_vmcnt<0>();  // copies issued past the last step must not land in the output tile
-    __syncthreads();  // K/V slots are dead: reuse their LDS for the output tile
+    ks_.drain();  // K/V slots are dead and no copy is in flight: reuse their LDS for the output tile
     T* o_lds = reinterpret_cast<T*>(smem) + wave * 32 * OS;
 #pragma unroll
     for (int db = 0; db < C::DB; db++) {

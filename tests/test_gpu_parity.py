@@ -81,6 +81,9 @@ def test_hip_library_is_the_backend(gpu_device):
 
 SHAPES = [  # B, M, N, H
     (2, 128, 128, 2), (1, 256, 320, 3), (1, 100, 77, 2), (1, 1, 1, 1), (1, 129, 257, 1), (1, 33, 500, 2),
+    # rows of whole 16-byte chunks (the copy path of the bias) with ragged tiles on both axes, and
+    # enough blocks for every LDS ring to wrap several times
+    (1, 150, 200, 2), (1, 300, 1000, 1),
 ]
 
 

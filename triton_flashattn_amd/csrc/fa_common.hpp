@@ -157,6 +157,14 @@ __device__ __forceinline__ void g2lds16_untracked(const void* src, void* lds_bas
         : "v"(src), "s"(lds_addr)
         : "memory");
 }
+// A wave-uniform pointer, forced into scalar registers (the compiler may have computed it with
+// vector instructions, and an inline-asm scalar operand is not moved there by itself).
+__device__ __forceinline__ uint64_t uniform_ptr(const void* p) {
+    const uint64_t b = (uint64_t)(uintptr_t)p;
+    const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)b);
+    const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(b >> 32));
+    return ((uint64_t)hi << 32) | lo;
+}
 // The same with a wave-uniform base and a 32-bit byte offset per lane.
 __device__ __forceinline__ void g2lds16_untracked(const void* base, unsigned voff, void* lds_base) {
     const unsigned lds_addr = __builtin_amdgcn_readfirstlane(
@@ -170,7 +178,7 @@ __device__ __forceinline__ void g2lds16_untracked(const void* base, unsigned vof
         "s_nop 0\n\t"
         "s_mov_b32 m0, %0"
         : "=&s"(saved_m0)
-        : "v"(voff), "s"(base), "s"(lds_addr)
+        : "v"(voff), "s"(uniform_ptr(base)), "s"(lds_addr)
         : "memory");
 }
 // global_load_lds_dword: lane l copies the 4 bytes at base + voff (per lane) to lds_base + 4 l
@@ -186,7 +194,7 @@ __device__ __forceinline__ void g2lds4_untracked(const void* base, unsigned voff
         "s_nop 0\n\t"
         "s_mov_b32 m0, %0"
         : "=&s"(saved_m0)
-        : "v"(voff), "s"(base), "s"(lds_addr)
+        : "v"(voff), "s"(uniform_ptr(base)), "s"(lds_addr)
         : "memory");
 }
 // s_waitcnt vmcnt(n) alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14, the other counters maxed)

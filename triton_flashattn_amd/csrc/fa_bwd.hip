@@ -48,8 +48,15 @@ __global__ __launch_bounds__(256) void fa_bwd_prep_kernel(const BwdParams p) {
 // dQ^T += K^T dS^T wants as its B operand.  K, V and the bias slices arrive through the same
 // counted direct-to-LDS copy rings as in the forward kernel.  Replaces _attn_bwd_dq
 // (flash_attention.py:458-646).
-template <typename T, int D, int BIAS, bool CAUSAL>
+//
+// FROM_DS: when the key-tile kernel has just written dBias in the element type of q, that tensor IS
+// dS rounded exactly as the reference rounds it before this product (flash_attention.py:516-520).
+// The kernel then reads the dBias slices through the bias ring instead of the bias, skips both
+// recomputed products, the exponentials and the V rows, and is one product instead of three.
+template <typename T, int D, int BIAS, bool CAUSAL, bool FROM_DS = false>
 __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_dq_kernel(const BwdParams p) {
+    static_assert(!FROM_DS || (BIAS == 2 && __is_same(T, _Float16)) || (BIAS == 3 && __is_same(T, __bf16)),
+                  "dS can stand in for the recomputation only in the element type of q");
     typedef StreamCfg<D, BIAS> C;
     typedef Swz<D> SW;
     typedef typename VecOf<T>::v8 T8;
@@ -77,6 +84,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_
     const T* vp = reinterpret_cast<const T*>(p.v) + (int64_t)b * p.sv.b + (int64_t)h * p.sv.h;
     const E* bp = nullptr;
     if (BIAS != 0) bp = reinterpret_cast<const E*>(p.bias) + (int64_t)b * p.sbias.b + (int64_t)h * p.sbias.h;
+    if (FROM_DS) bp = reinterpret_cast<const E*>(p.dbias) + (int64_t)b * p.sdbias.b + (int64_t)h * p.sdbias.h;
 
     // Q^T and dO^T as B operands: column my_m, k = d
     const T* dop = reinterpret_cast<const T*>(p.dout) + (int64_t)b * p.sdo.b + (int64_t)h * p.sdo.h;
@@ -84,7 +92,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_
 #pragma unroll
     for (int ks = 0; ks < C::KSTEPS; ks++) {
         i32x4 rq = {0, 0, 0, 0}, rd = {0, 0, 0, 0};
-        if (my_m < M) {
+        if (!FROM_DS && my_m < M) {
             rq = gld16(qp + (int64_t)my_m * p.sq.s + ks * 16 + 8 * g);
             rd = gld16(dop + (int64_t)my_m * p.sdo.s + ks * 16 + 8 * g);
         }
@@ -93,7 +101,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_
     }
     // LSE (log2 units) and delta of this lane's query row
     float lse_i = 0.f, delta_i = 0.f;
-    if (my_m < M) {
+    if (!FROM_DS && my_m < M) {
         lse_i = p.lse[((int64_t)b * p.H + h) * M + my_m];
         delta_i = p.delta[((int64_t)b * p.H + h) * M + my_m];
     }
@@ -111,8 +119,9 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_
 #pragma unroll
         for (int i = 0; i < 16; i++) dq_acc[db][i] = 0.f;
 
-    KeyStream<T, D, BIAS> ks_;
-    ks_.init(smem, kp, vp, bp, p.sk.s, p.sv.s, p.sbias.m, p.sbias.n, M, N, mw, wave, lane);
+    KeyStream<T, D, BIAS, !FROM_DS> ks_;
+    ks_.init(smem, kp, vp, bp, p.sk.s, p.sv.s, FROM_DS ? p.sdbias.m : p.sbias.m, FROM_DS ? p.sdbias.n : p.sbias.n, M, N,
+             mw, wave, lane);
 
     // One step of the K/V stream.  Interior steps (every key in range and visible to every row of
     // the work-group) run with STEP_MASKED = false: no range checks, no mask arithmetic.  BV: the
@@ -134,6 +143,23 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_
             // blocks entirely above this wave's diagonal or past the last key contribute nothing
             if (STEP_MASKED && ((CAUSAL && n0 + nh > mw + 31) || n0 + nh >= N)) continue;
             const bool need_mask = STEP_MASKED && ((n0 + nh + 32 > N) || (CAUSAL && n0 + nh + 31 > mw));
+            T8 dsb[2];
+            if constexpr (FROM_DS) {
+                // dS^T of the block straight from the dBias slice: 4 consecutive keys per read, in
+                // accumulator order; keys past N hold whatever column 0 holds and count as zero
+#pragma unroll
+                for (int q4 = 0; q4 < 4; q4++) {
+                    const int nl = 8 * q4 + 4 * g;
+                    T4 hv = *reinterpret_cast<const T4*>(b_lds + ks_.b_off(r, nl));
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const int i = q4 * 4 + e;
+                        T val = hv[e];
+                        if (STEP_MASKED && n0 + nh + nl + e >= N) val = (T)0.f;
+                        dsb[i >> 3][i & 7] = val;
+                    }
+                }
+            } else {
 
             // ---- S^T = K Q^T : s[i] is key n0 + nh + 8 (i/4) + 4 g + i%4, query my_m ----
             f32x16 s;
@@ -157,7 +183,6 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_
 
             // ---- P = 2^(S*scale + bias - LSE), dS = P (dP - delta) (flash_attention.py:497-517).
             // Masked tiles follow the reference's additive -1e6 arithmetic term by term.
-            T8 dsb[2];
             auto ds_step = [&](auto masked_tag) {
                 constexpr bool MASKED = decltype(masked_tag)::value;
 #pragma unroll
@@ -212,6 +237,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_
             } else {
                 ds_step(std::false_type{});
             }
+            }
 
             // ---- dQ^T += K^T dS^T : A = K^T gathered down the columns of the K tile ----
 #pragma unroll
@@ -237,7 +263,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_
 #pragma unroll 1
         for (int k = n_fast; k < n_steps; k++) kv_step(k, std::true_type{}, bv_tag);
     };
-    if (BIAS != 0 && p.bias_vec) run(std::true_type{});
+    if (FROM_DS || (BIAS != 0 && p.bias_vec)) run(std::true_type{});
     else run(std::false_type{});
 
     // ---- epilogue: dq = dQ * sm_scale (flash_attention.py:644-646) ----
@@ -787,6 +813,14 @@ template <typename T, int D> static hipError_t launch_all(const BwdParams& p, in
     }
     if (stages & 4) {
         dim3 qgrid((unsigned)(p.n_mtiles * p.B * p.H));
+        // dBias in the element type of q, written a moment ago by the key-tile kernel in rows of whole
+        // 16-byte chunks, is the dS the dQ product needs
+        constexpr int DS_BIAS = __is_same(T, _Float16) ? 2 : 3;
+        if (dbias && bias == DS_BIAS && p.dbias_vec) {
+            if (causal) hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, DS_BIAS, true, true>), qgrid, dim3(256), 0, st, p);
+            else hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, DS_BIAS, false, true>), qgrid, dim3(256), 0, st, p);
+            return hipGetLastError();
+        }
 #define FA_CASE(BK)                                                                                               \
     case BK:                                                                                                      \
         if (causal) hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, BK, true>), qgrid, dim3(256), 0, st, p);           \

@@ -278,7 +278,8 @@ template <int D, int BIAS> struct StreamCfg {
 // The copy machinery of the kernels tiled by StreamCfg (forward, dQ): one object per thread.
 // Completion of the copies is counted by hand: they complete in issue order and every wave issues
 // the same number every step, also past the last step (clamped rows, never used).
-template <typename T, int D, int BIAS> struct KeyStream {
+// WITH_V = false leaves the V rows out (a kernel that only needs K).
+template <typename T, int D, int BIAS, bool WITH_V = true> struct KeyStream {
     typedef StreamCfg<D, BIAS> C;
     typedef Swz<D> SW;
     typedef typename BiasElem<BIAS>::type E;
@@ -340,7 +341,7 @@ template <typename T, int D, int BIAS> struct KeyStream {
                 vo = (unsigned)(row * (int)sv * 2 + src * 16);
             }
             g2lds16_untracked(kt, ko, k_dst + c_idx[i] * 1024);
-            g2lds16_untracked(vt, vo, v_dst + c_idx[i] * 1024);
+            if constexpr (WITH_V) g2lds16_untracked(vt, vo, v_dst + c_idx[i] * 1024);
         }
     }
     // Bias slice of this wave for step k (32 rows x 32 keys) -> ring slot k % NBS.  Position c =
@@ -379,7 +380,7 @@ template <typename T, int D, int BIAS> struct KeyStream {
     // them, and issue the copies that go into the slots step k - 1 has just left.
     template <bool BV> __device__ __forceinline__ void begin_step(int k) {
         static_assert(BIAS == 0 || C::LA < C::NBS - 1, "the bias slice of a step must be issued before its K/V rows");
-        constexpr int OPS = 2 * C::KD + (BV ? C::BCH : 0);  // copies per wave per step
+        constexpr int OPS = (WITH_V ? 2 : 1) * C::KD + (BV ? C::BCH : 0);  // copies per wave per step
         // K/V of this step were issued LA steps ago; the bias copies issued right after them and
         // the copies of the steps since may still be in flight
         wait_vmcnt<(BV ? C::BCH : 0) + OPS*(C::LA - 1)>();

@@ -141,7 +141,10 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_
             const int nh = nb * 32;  // first key of this block inside the step
             __builtin_amdgcn_sched_barrier(0);  // keep the blocks apart
             // blocks entirely above this wave's diagonal or past the last key contribute nothing
-            if (STEP_MASKED && ((CAUSAL && n0 + nh > mw + 31) || n0 + nh >= N)) continue;
+            if (STEP_MASKED && ((CAUSAL && n0 + nh > mw + 31) || n0 + nh >= N)) {
+                if (nb == 0) ks_.template issue_ahead<BV>(k);  // every wave issues its copies in every step
+                continue;
+            }
             const bool need_mask = STEP_MASKED && ((n0 + nh + 32 > N) || (CAUSAL && n0 + nh + 31 > mw));
             T8 dsb[2];
             if constexpr (FROM_DS) {
@@ -180,6 +183,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_
                 T8 a = as_vec<T8>(lds_read16(v_lds + SW::off(nh + r, ks * 16 + 8 * g)));
                 dp = mfma32(a, doreg[ks], dp);
             }
+            if (nb == 0) ks_.template issue_ahead<BV>(k);  // in the shadow of the MFMAs just issued
 
             // ---- P = 2^(S*scale + bias - LSE), dS = P (dP - delta) (flash_attention.py:497-517).
             // Masked tiles follow the reference's additive -1e6 arithmetic term by term.
@@ -248,6 +252,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_
                     dq_acc[db] = mfma32(a, dsb[kk], dq_acc[db]);
                 }
             }
+            if (FROM_DS && nb == 0) ks_.template issue_ahead<BV>(k);  // in the shadow of the MFMAs just issued
         }
     };
 

@@ -376,8 +376,8 @@ template <typename T, int D, int BIAS, bool WITH_V = true> struct KeyStream {
             if constexpr (BV) issue_bias(C::NBS - 1 - C::LA + i);
         }
     }
-    // Top of step k: wait for its K/V rows (and with them its bias slice, issued earlier), publish
-    // them, and issue the copies that go into the slots step k - 1 has just left.
+    // Top of step k: wait for its K/V rows (and with them its bias slice, issued earlier) and
+    // publish them.  The slots that step k - 1 read are free from here on.
     template <bool BV> __device__ __forceinline__ void begin_step(int k) {
         static_assert(BIAS == 0 || C::LA < C::NBS - 1, "the bias slice of a step must be issued before its K/V rows");
         constexpr int OPS = (WITH_V ? 2 : 1) * C::KD + (BV ? C::BCH : 0);  // copies per wave per step
@@ -385,8 +385,6 @@ template <typename T, int D, int BIAS, bool WITH_V = true> struct KeyStream {
         // the copies of the steps since may still be in flight
         wait_vmcnt<(BV ? C::BCH : 0) + OPS*(C::LA - 1)>();
         lds_barrier();
-        issue_kv(k + C::LA);
-        if constexpr (BV) issue_bias(k + C::NBS - 1);
         if constexpr (BIAS != 0 && !BV) {
             // unaligned bias rows or non-unit key stride: one element per lane per row
             if (lane < 32) {
@@ -399,6 +397,14 @@ template <typename T, int D, int BIAS, bool WITH_V = true> struct KeyStream {
                 }
             }
         }
+    }
+    // Once per step, anywhere after begin_step(k): the copies that go into the slots step k - 1 has
+    // left.  Issuing a copy holds the wave while the copies of the other waves drain through the
+    // CU's 64 bytes/clock copy path, so the best place is right behind a batch of MFMAs, whose
+    // execution then hides it; right after the barrier all waves would queue up at once.
+    template <bool BV> __device__ __forceinline__ void issue_ahead(int k) {
+        issue_kv(k + C::LA);
+        if constexpr (BV) issue_bias(k + C::NBS - 1);
     }
     // After the last step: nothing may land in LDS that is about to be reused.
     __device__ __forceinline__ void drain() {

@@ -101,7 +101,10 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_
         const int nh = nb * 32;  // first key of this block inside the step
         __builtin_amdgcn_sched_barrier(0);  // keep the blocks apart
         // blocks entirely above this wave's diagonal or past the last key contribute nothing
-        if (STEP_MASKED && ((CAUSAL && n0 + nh > mw + 31) || n0 + nh >= N)) continue;
+        if (STEP_MASKED && ((CAUSAL && n0 + nh > mw + 31) || n0 + nh >= N)) {
+            if (nb == 0) ks_.template issue_ahead<BV>(k);  // every wave issues its copies in every step
+            continue;
+        }
         const bool need_mask = STEP_MASKED && ((n0 + nh + 32 > N) || (CAUSAL && n0 + nh + 31 > mw));
 
         // ---- S^T = K Q^T : s[i] is key n0 + nh + 8 (i/4) + 4 g + i%4, query my_m ----
@@ -113,6 +116,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_
             T8 a = as_vec<T8>(lds_read16(k_lds + SW::off(nh + r, ks * 16 + 8 * g)));
             s = mfma32(a, qreg[ks], s);
         }
+        if (nb == 0) ks_.template issue_ahead<BV>(k);  // in the shadow of the MFMAs just issued
 
         // ---- online softmax step.  `masked` steps (ragged edge, causal diagonal) and a
         // non-positive scale follow the reference's arithmetic term by term: scaled score,

@@ -365,7 +365,8 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
     const int wave = tid >> 6, lane = tid & 63;
     const int r = lane & 31, g = lane >> 5;
     const bool s_wave = wave < 4;  // role
-    const int kb = wave & 3;       // 32-key block of this wave
+    const int kb = __builtin_amdgcn_readfirstlane(wave & 3);  // 32-key block of this wave (scalar)
+    const unsigned lds_base = lds_addr_of(smem);
 
     int nt, bh;
     decode_block(blockIdx.x, p.n_ntiles, p.B * p.H, nt, bh);
@@ -446,10 +447,10 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
         cq_off[i] = (unsigned)(row * (int)p.sq.s * 2 + src * 16);
         cdo_off[i] = (unsigned)(row * (int)p.sdo.s * 2 + src * 16);
     }
-    auto issue_rows = [&](const T* base, int64_t row_stride, const unsigned (&off)[C::QD], int mb, unsigned char* dst) {
+    auto issue_rows = [&](const T* base, int64_t row_stride, const unsigned (&off)[C::QD], int mb, unsigned dst) {
         // a block past the end is the last row over and over: offsets never go negative
         const int m0 = mb * BMI < M ? mb * BMI : M - 1;
-        const T* blk = base + (int64_t)m0 * row_stride;
+        const uint64_t blk = uniform_ptr(base + (int64_t)m0 * row_stride);
         const bool full = m0 + BMI <= M;
 #pragma unroll
         for (int i = 0; i < C::QD; i++) {
@@ -461,15 +462,15 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
                 row = row < M - m0 ? row : M - 1 - m0;
                 o = (unsigned)(row * (int)row_stride * 2 + src * 16);
             }
-            g2lds16_untracked(blk, o, dst + c_idx[i] * 1024);
+            lds_copy16(blk, o, dst + c_idx[i] * 1024);
         }
     };
-    // one float per row: the even S-waves copy LSE, the odd ones delta
-    auto issue_stat = [&](const float* src, int mb, float* dst) {
+    // one float per row
+    auto issue_stat = [&](const float* src, int mb, unsigned dst) {
         if (lane < BMI) {
             int m = mb * BMI + lane;
             m = m < M ? m : M - 1;
-            g2lds4_untracked(src, (unsigned)m * 4u, dst);
+            lds_copy4(uniform_ptr(src), (unsigned)m * 4u, dst);
         }
     };
     // bias slice (BMI rows x 32 keys) of query block mb -> ring slot.  Chunk c = 64 it + lane of the
@@ -478,7 +479,8 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
     // column 0: both are masked where they are used.
     auto issue_bias = [&](int mb) {
         if constexpr (BIAS != 0) {
-            unsigned char* dst = ring_lds + ((mb - mb_first) % C::RING) * C::BT_BYTES;
+            const unsigned dst = lds_base + C::OFF_BIAS + (kb * C::RING + (mb - mb_first) % C::RING) * C::BT_BYTES;
+            const uint64_t base = uniform_ptr(bp);
 #pragma unroll
             for (int it = 0; it < C::BCH; it++) {
                 const int c = it * 64 + lane;
@@ -486,19 +488,20 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
                 int nn = nw + (c % C::BCPR) * C::EPC;
                 m = m < M ? m : M - 1;
                 nn = nn < N ? nn : 0;
-                g2lds16_untracked(bp + (int64_t)m * p.sbias.m + nn, dst + it * 1024);
+                // a (batch, head) slice that takes this path is smaller than 2 GiB
+                lds_copy16(base, (unsigned)(((int64_t)m * p.sbias.m + nn) * C::ES), dst + it * 1024);
             }
         }
     };
     // block mb of Q with its LSE (QD + 1 copies) / block mb of dO with its delta (QD + 1 copies);
     // all four waves of a role copy the 32 or 64 floats, which keeps their counts alike
     auto issue_q = [&](int mb) {
-        issue_rows(qp, p.sq.s, cq_off, mb, smem + (mb % C::NQB) * C::Q_BYTES);
-        issue_stat(lsep, mb, reinterpret_cast<float*>(smem + C::OFF_LSE) + (mb % C::NQB) * BMI);
+        issue_rows(qp, p.sq.s, cq_off, mb, lds_base + (mb % C::NQB) * C::Q_BYTES);
+        issue_stat(lsep, mb, lds_base + C::OFF_LSE + (mb % C::NQB) * BMI * 4);
     };
     auto issue_do = [&](int mb) {
-        issue_rows(dop, p.sdo.s, cdo_off, mb, smem + C::OFF_DO + (mb % C::NDOB) * C::Q_BYTES);
-        issue_stat(deltap, mb, reinterpret_cast<float*>(smem + C::OFF_DELTA) + (mb % C::NDOB) * BMI);
+        issue_rows(dop, p.sdo.s, cdo_off, mb, lds_base + C::OFF_DO + (mb % C::NDOB) * C::Q_BYTES);
+        issue_stat(deltap, mb, lds_base + C::OFF_DELTA + (mb % C::NDOB) * BMI * 4);
     };
     // Issuing a copy stalls the wave while the memory pipeline of the CU is backed up, so the
     // copies are dealt out between the roles: Q and the bias go with the S-waves, dO with the
@@ -519,11 +522,15 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
     };
 
     // ---- prologue: the first LA blocks of Q and LA - 1 blocks of dO ----
+    {
+        const unsigned saved_m0 = lds_copy_begin();
 #pragma unroll 1
-    for (int i = 0; i < C::LA; i++) {
-        if (s_wave == Q_BY_S) issue_q(mb_first + i);
-        if (s_wave && BIAS != 0 && bias_vec) issue_bias(mb_first + i);
-        if (s_wave == DO_BY_S && i < C::LA - 1) issue_do(mb_first + i);
+        for (int i = 0; i < C::LA; i++) {
+            if (s_wave == Q_BY_S) issue_q(mb_first + i);
+            if (s_wave && BIAS != 0 && bias_vec) issue_bias(mb_first + i);
+            if (s_wave == DO_BY_S && i < C::LA - 1) issue_do(mb_first + i);
+        }
+        lds_copy_end(saved_m0);
     }
     wait_vmcnt<0>();
     __syncthreads();
@@ -571,9 +578,13 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
             const int nb = t + 1;  // the block whose P is produced in this step
             T8 op_next[NSUB][2];
             // copies for the steps to come; their buffers were last read one step ago
-            if constexpr (Q_BY_S) issue_q(nb + C::LA);
-            if constexpr (BV) issue_bias(nb + C::LA);
-            if constexpr (DO_BY_S) issue_do(t + C::LA);
+            {
+                const unsigned saved_m0 = lds_copy_begin();
+                if constexpr (Q_BY_S) issue_q(nb + C::LA);
+                if constexpr (BV) issue_bias(nb + C::LA);
+                if constexpr (DO_BY_S) issue_do(t + C::LA);
+                lds_copy_end(saved_m0);
+            }
             // dV^T += dO(t)^T P(t) first: its operands are ready, and the Q rows of the next block
             // can be on their way out of LDS meanwhile
             if (t >= mb_first && t < n_mblocks)
@@ -686,8 +697,12 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
         constexpr int COPIES = ((Q_BY_S ? 0 : 1) + (DO_BY_S ? 0 : 1)) * (C::QD + 1);
 #pragma unroll 1
         for (int t = mb_first - 1; t <= n_mblocks; t++) {
-            if constexpr (!Q_BY_S) issue_q(t + 1 + C::LA);
-            if constexpr (!DO_BY_S) issue_do(t + C::LA);
+            if constexpr (COPIES > 0) {
+                const unsigned saved_m0 = lds_copy_begin();
+                if constexpr (!Q_BY_S) issue_q(t + 1 + C::LA);
+                if constexpr (!DO_BY_S) issue_do(t + C::LA);
+                lds_copy_end(saved_m0);
+            }
             if (C::DEFER_DK && t - 1 >= mb_first)  // dK^T += Q(t-1)^T dS(t-1)
                 gemm_cols(reinterpret_cast<const T*>(smem + ((t - 1) % C::NQB) * C::Q_BYTES), op_cur);
             if (t >= mb_first && t < n_mblocks) {

@@ -129,33 +129,33 @@ template <int D> struct Swz {
 };
 
 // ---- global access ------------------------------------------------------------------------
-// global_load_lds_dwordx4: lane l copies the 16 bytes at `src` (per lane) to lds_base + 16 l
-// (lds_base is wave-uniform) without passing through registers; completion counts on vmcnt.
-__device__ __forceinline__ void g2lds16(const void* src, void* lds_base) {
-    __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1)))*)src,
-                                     (void __attribute__((address_space(3)))*)lds_base, 16, 0, 0);
-}
-
-// The same copy, issued behind the compiler's back.  The compiler makes every later LDS read that
-// might alias a direct-to-LDS copy wait for ALL outstanding vector-memory operations, which
-// empties a queue of copies issued several steps ahead.  Here it sees neither the LDS write nor
-// the vmcnt increment: the consumer must wait with an explicit s_waitcnt vmcnt(n) (copies
-// complete in issue order) before it reads the destination, and a wave that uses this must not
-// mix it with loads whose completion the compiler counts.  M0 is saved and restored.
-__device__ __forceinline__ void g2lds16_untracked(const void* src, void* lds_base) {
-    const unsigned lds_addr = __builtin_amdgcn_readfirstlane(
-        (unsigned)(uintptr_t)(__attribute__((address_space(3))) void*)lds_base);
+// Direct global -> LDS copies, issued behind the compiler's back.
+//
+// global_load_lds_dwordx4: lane l copies the 16 bytes at base + voff (voff per lane) to LDS address
+// M0 + 16 l, without passing through registers; completion counts on vmcnt.  Issued through the
+// compiler's builtin, every later LDS read that might alias the copy would wait for ALL
+// outstanding vector-memory operations, which empties a queue of copies issued several steps
+// ahead.  Issued from inline assembly the compiler sees neither the LDS write nor the vmcnt
+// increment: the consumer waits with an explicit s_waitcnt vmcnt(n) (copies complete in issue
+// order) before it reads the destination, and a wave that uses this must not mix it with loads
+// whose completion the compiler counts.
+//
+// A copy costs the issuing wave about 20 clocks when everything it needs is in scalar registers
+// (57 with M0 saved and restored around each one and the addresses moved over from vector
+// registers), so copies are issued in batches: M0 saved once, restored once, LDS addresses and
+// base pointers scalar.
+__device__ __forceinline__ unsigned lds_copy_begin() {
     unsigned saved_m0;
-    asm volatile(
-        "s_mov_b32 %0, m0\n\t"
-        "s_mov_b32 m0, %2\n\t"
-        "s_nop 0\n\t"
-        "global_load_lds_dwordx4 %1, off\n\t"
-        "s_nop 0\n\t"
-        "s_mov_b32 m0, %0"
-        : "=&s"(saved_m0)
-        : "v"(src), "s"(lds_addr)
-        : "memory");
+    asm volatile("s_mov_b32 %0, m0" : "=s"(saved_m0) : : "memory");
+    return saved_m0;
+}
+__device__ __forceinline__ void lds_copy_end(unsigned saved_m0) {
+    asm volatile("s_mov_b32 m0, %0" : : "s"(saved_m0) : "memory");
+}
+// the LDS address (scalar) of a generic pointer into LDS that is the same in every lane: the low
+// half of the generic pointer
+__device__ __forceinline__ unsigned lds_addr_of(const void* p) {
+    return __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)p);
 }
 // A wave-uniform pointer, forced into scalar registers (the compiler may have computed it with
 // vector instructions, and an inline-asm scalar operand is not moved there by itself).
@@ -165,36 +165,24 @@ __device__ __forceinline__ uint64_t uniform_ptr(const void* p) {
     const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(b >> 32));
     return ((uint64_t)hi << 32) | lo;
 }
-// The same with a wave-uniform base and a 32-bit byte offset per lane.
-__device__ __forceinline__ void g2lds16_untracked(const void* base, unsigned voff, void* lds_base) {
-    const unsigned lds_addr = __builtin_amdgcn_readfirstlane(
-        (unsigned)(uintptr_t)(__attribute__((address_space(3))) void*)lds_base);
-    unsigned saved_m0;
+// between lds_copy_begin() and lds_copy_end(): 16 bytes per lane from base + voff to lds_addr + 16 l
+__device__ __forceinline__ void lds_copy16(uint64_t base, unsigned voff, unsigned lds_addr) {
     asm volatile(
-        "s_mov_b32 %0, m0\n\t"
-        "s_mov_b32 m0, %3\n\t"
+        "s_mov_b32 m0, %2\n\t"
         "s_nop 0\n\t"
-        "global_load_lds_dwordx4 %1, %2\n\t"
-        "s_nop 0\n\t"
-        "s_mov_b32 m0, %0"
-        : "=&s"(saved_m0)
-        : "v"(voff), "s"(uniform_ptr(base)), "s"(lds_addr)
+        "global_load_lds_dwordx4 %0, %1"
+        :
+        : "v"(voff), "s"(base), "s"(lds_addr)
         : "memory");
 }
-// global_load_lds_dword: lane l copies the 4 bytes at base + voff (per lane) to lds_base + 4 l
-__device__ __forceinline__ void g2lds4_untracked(const void* base, unsigned voff, void* lds_base) {
-    const unsigned lds_addr = __builtin_amdgcn_readfirstlane(
-        (unsigned)(uintptr_t)(__attribute__((address_space(3))) void*)lds_base);
-    unsigned saved_m0;
+// the same for 4 bytes per lane, to lds_addr + 4 l
+__device__ __forceinline__ void lds_copy4(uint64_t base, unsigned voff, unsigned lds_addr) {
     asm volatile(
-        "s_mov_b32 %0, m0\n\t"
-        "s_mov_b32 m0, %3\n\t"
+        "s_mov_b32 m0, %2\n\t"
         "s_nop 0\n\t"
-        "global_load_lds_dword %1, %2\n\t"
-        "s_nop 0\n\t"
-        "s_mov_b32 m0, %0"
-        : "=&s"(saved_m0)
-        : "v"(voff), "s"(uniform_ptr(base)), "s"(lds_addr)
+        "global_load_lds_dword %0, %1"
+        :
+        : "v"(voff), "s"(base), "s"(lds_addr)
         : "memory");
 }
 // s_waitcnt vmcnt(n) alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14, the other counters maxed)
@@ -292,6 +280,7 @@ template <typename T, int D, int BIAS, bool WITH_V = true> struct KeyStream {
     int M, N, mw, lane;
     unsigned k_off[C::KD], v_off[C::KD];
     int c_idx[C::KD];
+    unsigned lds_kv, lds_bias;  // LDS addresses (scalar) of the K slots and of this wave's bias ring
 
     // K / V rows of a step: NKD copies of 1 KB each; copy ci fills bytes [1024 ci, 1024 ci + 1024) of
     // the swizzled slot, so lane l of it fetches the chunk that lives at slot position 64 ci + l
@@ -301,7 +290,10 @@ template <typename T, int D, int BIAS, bool WITH_V = true> struct KeyStream {
                                          int64_t sv_, int64_t sbm_, int64_t sbn_, int M_, int N_, int mw_, int wave, int lane_) {
         smem = smem_; kp = kp_; vp = vp_; bp = bp_; sk = sk_; sv = sv_; sbm = sbm_; sbn = sbn_;
         M = M_; N = N_; mw = mw_; lane = lane_;
+        wave = __builtin_amdgcn_readfirstlane(wave);  // the same in every lane: keep it scalar
         bias_lds = smem + C::KV_BYTES + wave * C::NBS * C::BSLOT;
+        lds_kv = lds_addr_of(smem);
+        lds_bias = lds_kv + C::KV_BYTES + wave * C::NBS * C::BSLOT;
 #pragma unroll
         for (int i = 0; i < C::KD; i++) {
             c_idx[i] = (wave * C::KD + i) % C::NKD;
@@ -324,10 +316,10 @@ template <typename T, int D, int BIAS, bool WITH_V = true> struct KeyStream {
     // over and over, so that offsets never go negative.
     __device__ __forceinline__ void issue_kv(int k) {
         const int n0 = k * C::BK < N ? k * C::BK : N - 1;
-        const T* kt = kp + (int64_t)n0 * sk;
-        const T* vt = vp + (int64_t)n0 * sv;
-        unsigned char* k_dst = smem + (k % C::NKV) * C::STEP_BYTES;
-        unsigned char* v_dst = smem + (C::NKV + k % C::NKV) * C::STEP_BYTES;
+        const uint64_t kt = uniform_ptr(kp + (int64_t)n0 * sk);
+        const uint64_t vt = uniform_ptr(vp + (int64_t)n0 * sv);
+        const unsigned k_dst = lds_kv + (k % C::NKV) * C::STEP_BYTES;
+        const unsigned v_dst = lds_kv + (C::NKV + k % C::NKV) * C::STEP_BYTES;
         const bool full = n0 + C::BK <= N;
 #pragma unroll
         for (int i = 0; i < C::KD; i++) {
@@ -340,8 +332,8 @@ template <typename T, int D, int BIAS, bool WITH_V = true> struct KeyStream {
                 ko = (unsigned)(row * (int)sk * 2 + src * 16);
                 vo = (unsigned)(row * (int)sv * 2 + src * 16);
             }
-            g2lds16_untracked(kt, ko, k_dst + c_idx[i] * 1024);
-            if constexpr (WITH_V) g2lds16_untracked(vt, vo, v_dst + c_idx[i] * 1024);
+            lds_copy16(kt, ko, k_dst + c_idx[i] * 1024);
+            if constexpr (WITH_V) lds_copy16(vt, vo, v_dst + c_idx[i] * 1024);
         }
     }
     // Bias slice of this wave for step k (32 rows x 32 keys) -> ring slot k % NBS.  Position c =
@@ -350,7 +342,8 @@ template <typename T, int D, int BIAS, bool WITH_V = true> struct KeyStream {
     // re-read column 0 (masked).
     __device__ __forceinline__ void issue_bias(int k) {
         if constexpr (BIAS != 0) {
-            unsigned char* dst = b_lds(k);
+            const unsigned dst = lds_bias + (k % C::NBS) * C::BSLOT;
+            const uint64_t base = uniform_ptr(bp);
 #pragma unroll
             for (int it = 0; it < C::BCH; it++) {
                 const int c = it * 64 + lane;
@@ -359,13 +352,15 @@ template <typename T, int D, int BIAS, bool WITH_V = true> struct KeyStream {
                 int n = k * C::BK + ((c % C::BCPR) ^ C::bswz(row)) * C::EPC;
                 m = m < M ? m : M - 1;
                 n = n < N ? n : 0;
-                g2lds16_untracked(bp + (int64_t)m * sbm + n, dst + it * 1024);
+                // a (batch, head) slice that takes this path is smaller than 2 GiB
+                lds_copy16(base, (unsigned)(((int64_t)m * sbm + n) * C::ES), dst + it * 1024);
             }
         }
     }
     // Before the first step, in the order the steps assume: the first bias slices, then K/V of a
     // step followed by the bias slice issued in the same step.  BV: the bias slices come by copy.
     template <bool BV> __device__ __forceinline__ void prologue() {
+        const unsigned saved_m0 = lds_copy_begin();
         if constexpr (BV) {
 #pragma unroll
             for (int i = 0; i < C::NBS - 1 - C::LA; i++) issue_bias(i);
@@ -375,6 +370,7 @@ template <typename T, int D, int BIAS, bool WITH_V = true> struct KeyStream {
             issue_kv(i);
             if constexpr (BV) issue_bias(C::NBS - 1 - C::LA + i);
         }
+        lds_copy_end(saved_m0);
     }
     // Top of step k: wait for its K/V rows (and with them its bias slice, issued earlier) and
     // publish them.  The slots that step k - 1 read are free from here on.
@@ -403,8 +399,10 @@ template <typename T, int D, int BIAS, bool WITH_V = true> struct KeyStream {
     // CU's 64 bytes/clock copy path, so the best place is right behind a batch of MFMAs, whose
     // execution then hides it; right after the barrier all waves would queue up at once.
     template <bool BV> __device__ __forceinline__ void issue_ahead(int k) {
+        const unsigned saved_m0 = lds_copy_begin();
         issue_kv(k + C::LA);
         if constexpr (BV) issue_bias(k + C::NBS - 1);
+        lds_copy_end(saved_m0);
     }
     // After the last step: nothing may land in LDS that is about to be reused.
     __device__ __forceinline__ void drain() {

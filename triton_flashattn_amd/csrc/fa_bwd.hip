@@ -577,18 +577,22 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
         for (int t = mb_first - 1; t <= n_mblocks; t++) {
             const int nb = t + 1;  // the block whose P is produced in this step
             T8 op_next[NSUB][2];
-            // copies for the steps to come; their buffers were last read one step ago
-            {
+            // Copies for the steps to come (their buffers were last read one step ago).  With a bias
+            // they are issued in the shadow of the first MFMAs of the step, without one right
+            // after the barrier: measured, each way is a few per cent better in its case.
+            auto issue_copies = [&]() {
                 const unsigned saved_m0 = lds_copy_begin();
                 if constexpr (Q_BY_S) issue_q(nb + C::LA);
                 if constexpr (BV) issue_bias(nb + C::LA);
                 if constexpr (DO_BY_S) issue_do(t + C::LA);
                 lds_copy_end(saved_m0);
-            }
+            };
+            if constexpr (BIAS == 0) issue_copies();
             // dV^T += dO(t)^T P(t) first: its operands are ready, and the Q rows of the next block
             // can be on their way out of LDS meanwhile
             if (t >= mb_first && t < n_mblocks)
                 gemm_cols(reinterpret_cast<const T*>(smem + C::OFF_DO + (t % C::NDOB) * C::Q_BYTES), op_cur);
+            if constexpr (BIAS != 0) issue_copies();
             if (nb < n_mblocks) {
                 const int m0 = nb * BMI;
                 const unsigned char* bt_lds = ring_lds + ((nb - mb_first) % C::RING) * C::BT_BYTES;
@@ -697,14 +701,18 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
         constexpr int COPIES = ((Q_BY_S ? 0 : 1) + (DO_BY_S ? 0 : 1)) * (C::QD + 1);
 #pragma unroll 1
         for (int t = mb_first - 1; t <= n_mblocks; t++) {
-            if constexpr (COPIES > 0) {
-                const unsigned saved_m0 = lds_copy_begin();
-                if constexpr (!Q_BY_S) issue_q(t + 1 + C::LA);
-                if constexpr (!DO_BY_S) issue_do(t + C::LA);
-                lds_copy_end(saved_m0);
-            }
+            auto issue_copies = [&]() {
+                if constexpr (COPIES > 0) {
+                    const unsigned saved_m0 = lds_copy_begin();
+                    if constexpr (!Q_BY_S) issue_q(t + 1 + C::LA);
+                    if constexpr (!DO_BY_S) issue_do(t + C::LA);
+                    lds_copy_end(saved_m0);
+                }
+            };
+            if constexpr (BIAS == 0) issue_copies();
             if (C::DEFER_DK && t - 1 >= mb_first)  // dK^T += Q(t-1)^T dS(t-1)
                 gemm_cols(reinterpret_cast<const T*>(smem + ((t - 1) % C::NQB) * C::Q_BYTES), op_cur);
+            if constexpr (BIAS != 0) issue_copies();  // in the shadow of the MFMAs just issued
             if (t >= mb_first && t < n_mblocks) {
                 const int m0 = t * BMI;
                 f32x16 sacc[NSUB];

@@ -73,7 +73,6 @@ __device__ __forceinline__ void lds_barrier() {
 
 // ---- LDS access ---------------------------------------------------------------------------
 __device__ __forceinline__ i32x4 lds_read16(const void* p) { return *reinterpret_cast<const i32x4*>(p); }
-__device__ __forceinline__ void lds_write16(void* p, i32x4 v) { *reinterpret_cast<i32x4*>(p) = v; }
 
 // ds_read_b64_tr_b16.  Within each group of 16 lanes, lane s supplies the address of four
 // consecutive 16-bit elements: row s/4, columns 4*(s%4) .. 4*(s%4)+3 of a 4 x 16 matrix.  Lane i
@@ -89,18 +88,6 @@ __device__ __forceinline__ int tr_offset(int lane, int row0, int col0, int strid
     int s = lane & 15;
     return (row0 + (s >> 2)) * stride + col0 + ((lane >> 4) & 1) * 16 + (s & 3) * 4;
 }
-// 8 k-slots of an A/B operand gathered down a column of a row-major LDS tile: rows
-// row0 + 4g + {0..3} and row0 + 8 + 4g + {0..3} (g = lane/32), column col0 + lane%32.
-template <typename V8, typename T>
-__device__ __forceinline__ V8 lds_read_col8(const T* tile, int lane, int row0, int col0, int stride) {
-    int g = lane >> 5;
-    i16x4 lo = lds_read_tr4(tile + tr_offset(lane, row0 + 4 * g, col0, stride));
-    i16x4 hi = lds_read_tr4(tile + tr_offset(lane, row0 + 8 + 4 * g, col0, stride));
-    typedef short i16x8 __attribute__((ext_vector_type(8)));
-    i16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    return __builtin_bit_cast(V8, v);
-}
-
 // Row-major LDS tile of 16-bit elements, D per row, no padding; the 16-byte chunks of a row are
 // XOR-swizzled by a function of the row so that both 16-byte row reads (lane = row) and 4-row
 // column gathers (ds_read_b64_tr_b16) are free of bank conflicts.
@@ -190,8 +177,8 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() {
     __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
 }
 
-// Raw buffer view of `bytes` bytes at `base` (16-byte aligned): loads beyond the end return 0 and
-// stores beyond the end are dropped.  The range check works on whole dwords, so the length is
+// Raw buffer view of `bytes` bytes at `base` (16-byte aligned): stores beyond the end are dropped
+// (and loads beyond it would return 0).  The range check works on whole dwords, so the length is
 // rounded up to the dword that holds the last byte (still inside the aligned allocation); a
 // caller that stores through the view must not address the rounding slack.
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_buffer(const void* base, int64_t bytes) {
@@ -204,17 +191,8 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_buffer(const void* base, 
 __device__ __forceinline__ void buf_store16(__amdgpu_buffer_rsrc_t r, i32x4 v, int voff) {
     __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(__attribute__((__vector_size__(4 * sizeof(unsigned int)))) unsigned int, v), r, voff, 0, 0);
 }
-__device__ __forceinline__ float buf_load_f32(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
-}
-__device__ __forceinline__ i32x4 buf_load16(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
-    return __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
-}
-
 __device__ __forceinline__ i32x4 gld16(const void* p) { return *reinterpret_cast<const i32x4*>(p); }
 __device__ __forceinline__ void gst16(void* p, i32x4 v) { *reinterpret_cast<i32x4*>(p) = v; }
-
-template <typename T> __device__ __forceinline__ float to_f32(T x) { return (float)x; }
 
 // bias element -> fp32 (natural units); E is the storage type selected by the bias kind
 template <int BIAS> struct BiasElem;

@@ -51,7 +51,7 @@ def run_ours(q, k, v, do, bias, causal, sm_scale=None):
     out = flash_attention_fn(q, k, v, bias, causal, sm_scale)
     out.backward(do)
     res = {"out": out.detach(), "dq": q.grad, "dk": k.grad, "dv": v.grad, "dbias": None}
-    if bias is not None and bias.requires_grad:
+    if bias is not None and bias.requires_grad and bias.is_leaf:
         res["dbias"] = bias.grad
         bias.grad = None
     return res
@@ -289,6 +289,32 @@ def test_noncontiguous_inputs_and_upstream_grad(gpu_device):
     ref = run_oracle(qs, ks, v, dos, bias_t, False)
     check(ours, ref, "strided")
     assert ours["dbias"].shape == bias_t.shape
+
+
+def test_bias_layouts(gpu_device):
+    """Biases that are not dense (B, H, M, N) tensors of the dtype of q: rows padded to a wider
+    stride, a broadcast (1, H, 1, N) bias whose gradient autograd reduces, and a trainable bias of
+    the other 16-bit type (dBias then cannot stand in for dS in the dQ kernel)."""
+    B, M, N, H, D = 2, 200, 328, 2, 64
+    for dtype, causal in ((torch.bfloat16, False), (torch.float16, False), (torch.bfloat16, True)):
+        n = M if causal else N
+        q, k, v, do, _ = make_inputs(gpu_device, B, M, n, H, D, dtype, None, seed=5)
+        g = torch.Generator(device="cpu").manual_seed(6)
+        mk = lambda *s_, dt=dtype: torch.randn(*s_, generator=g).to(dt).to(gpu_device)
+        other = torch.float16 if dtype == torch.bfloat16 else torch.bfloat16
+        leaf_b = mk(1, H, 1, n).requires_grad_(True)
+        cases = {
+            "padded rows": (mk(B, H, M, n + 24)[..., :n].detach().requires_grad_(True), None),
+            "broadcast": (leaf_b.expand(B, H, M, n), leaf_b),
+            "other 16-bit type": (mk(B, H, M, n, dt=other).requires_grad_(True), None),
+        }
+        for name, (bias, leaf) in cases.items():
+            ours = run_ours(q, k, v, do, bias, causal)
+            ref = run_oracle(q, k, v, do, bias, causal)
+            if leaf is not None:
+                ours["dbias"], leaf.grad = leaf.grad, None
+                ref["dbias"] = ref["dbias"].sum_to_size(leaf.shape)
+            check(ours, ref, "%s %s causal=%s" % (name, dtype, causal))
 
 
 def test_repeatability(gpu_device):

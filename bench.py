@@ -64,11 +64,13 @@ def make_config(name, dev):
         return dict(q=rn(B, M, H, D), k=rn(B, N, H, D), v=rn(B, N, H, D), do=rn(B, M, H, D),
                     bias=rn(B, H, M, N).requires_grad_(True), causal=False, dims=(B, H, M, N, D), bias_es=2,
                     trainable=True)
-    if name == "C4":
+    if name in ("C4", "C4_expanded_mask"):
         B, S, H, D = 8, 1024, 12, 64
         qkv = rn(B, S, 3, H, D)
         lens = torch.randint(512, 1025, (B,), device=dev, generator=g)
-        keep = (torch.arange(S, device=dev)[None, :] < lens[:, None])[:, None, None, :].expand(B, H, S, S).contiguous()
+        keep = (torch.arange(S, device=dev)[None, :] < lens[:, None])[:, None, None, :].expand(B, H, S, S)
+        if name == "C4":
+            keep = keep.contiguous()  # the number of record; the other one reads the (B,1,1,S) mask in place
         return dict(q=qkv[:, :, 0], k=qkv[:, :, 1], v=qkv[:, :, 2], do=rn(B, S, H, D), bias=keep, causal=True,
                     dims=(B, H, S, S, D), bias_es=1, trainable=False)
     if name == "C5":
@@ -253,7 +255,7 @@ def main():
 
     if not args.no_other_configs:
         others = {}
-        for name in ("C2", "C4", "C5"):
+        for name in ("C2", "C4", "C4_expanded_mask", "C5"):
             del cfg
             torch.cuda.empty_cache()
             cfg = make_config(name, dev)

@@ -615,7 +615,8 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
                         for (int q4 = 0; q4 < 4; q4++) {
                             const int ml0 = sb * 32 + 8 * q4 + 4 * g;  // first of 4 consecutive rows
                             const f32x4 lse4 = *reinterpret_cast<const f32x4*>(lse_lds + ml0);
-                            float bv[4] = {0.f, 0.f, 0.f, 0.f};  // bias in log2 units / mask term
+                            // bool mask: the additive term in log2 units; float bias: natural units
+                            float bv[4] = {0.f, 0.f, 0.f, 0.f};
                             if constexpr (BIAS == 1) {
 #pragma unroll
                                 for (int e = 0; e < 4; e++) bv[e] = bt_lds[(ml0 + e) * 32 + r] ? 0.f : kMask;
@@ -624,11 +625,10 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
                                 i16x4 raw = lds_read_tr4(reinterpret_cast<const E*>(bt_lds) + tr_offset(lane, ml0, 0, 32));
                                 B4 hv = __builtin_bit_cast(B4, raw);
 #pragma unroll
-                                for (int e = 0; e < 4; e++) bv[e] = (float)hv[e] * kLog2e;
+                                for (int e = 0; e < 4; e++) bv[e] = (float)hv[e];
                             } else if constexpr (BIAS == 4) {
 #pragma unroll
-                                for (int e = 0; e < 4; e++)
-                                    bv[e] = reinterpret_cast<const float*>(bt_lds)[(ml0 + e) * 32 + r] * kLog2e;
+                                for (int e = 0; e < 4; e++) bv[e] = reinterpret_cast<const float*>(bt_lds)[(ml0 + e) * 32 + r];
                             }
                             f32x4 p4;
 #pragma unroll
@@ -641,12 +641,13 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
                                     const bool oob = (m >= M) || (my_n >= N);
                                     float tmask = oob ? kMask : 0.f;
                                     if (CAUSAL) tmask += (m < my_n) ? kMask : 0.f;
-                                    float add = bv[e];
+                                    float add = BIAS >= 2 ? __fmul_rn(bv[e], kLog2e) : bv[e];
                                     if (BIAS != 0) add = oob ? kMask : add;
                                     x = __fadd_rn(x, __fadd_rn(tmask, add));
                                     pv = fast_exp2(x - lse4[e]);
                                 } else {
-                                    pv = fast_exp2(__builtin_fmaf(sacc[sb][i], qk_scale, bv[e] - lse4[e]));
+                                    const float off = BIAS >= 2 ? __builtin_fmaf(bv[e], kLog2e, -lse4[e]) : bv[e] - lse4[e];
+                                    pv = fast_exp2(__builtin_fmaf(sacc[sb][i], qk_scale, off));
                                 }
                                 p4[e] = pv;
                                 op_next[sb][i >> 3][i & 7] = (T)pv;

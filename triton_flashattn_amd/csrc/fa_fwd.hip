@@ -94,8 +94,24 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_
         const T* v_lds = ks_.v_lds(k);
         const unsigned char* b_lds = ks_.b_lds(k);
         static_assert(BIAS == 0 || C::NH == 1, "a bias slot covers one 32-key block");
-        // The step is consumed 32 keys at a time, each block with its own softmax step, so that only
-        // one 32 x 32 score block is live at a time.
+        // The step is consumed 32 keys at a time, each block with its own softmax step.  In interior
+        // steps of more than one block all score products are issued up front: the MFMAs of the later
+        // blocks then run while the vector pipeline works on the first.
+        constexpr bool PRE = !STEP_MASKED && C::NH > 1;
+        f32x16 s_pre[C::NH];
+        if constexpr (PRE) {
+#pragma unroll
+            for (int nb = 0; nb < C::NH; nb++) {
+#pragma unroll
+                for (int i = 0; i < 16; i++) s_pre[nb][i] = 0.f;
+#pragma unroll
+                for (int ks = 0; ks < C::KSTEPS; ks++) {
+                    T8 a = as_vec<T8>(lds_read16(k_lds + SW::off(nb * 32 + r, ks * 16 + 8 * g)));
+                    s_pre[nb] = mfma32(a, qreg[ks], s_pre[nb]);
+                }
+            }
+            ks_.template issue_ahead<BV>(k);  // in the shadow of the MFMAs just issued
+        }
 #pragma unroll
         for (int nb = 0; nb < C::NH; nb++) {
         const int nh = nb * 32;  // first key of this block inside the step
@@ -109,14 +125,18 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_
 
         // ---- S^T = K Q^T : s[i] is key n0 + nh + 8 (i/4) + 4 g + i%4, query my_m ----
         f32x16 s;
+        if constexpr (PRE) {
+            s = s_pre[nb];
+        } else {
 #pragma unroll
-        for (int i = 0; i < 16; i++) s[i] = 0.f;
+            for (int i = 0; i < 16; i++) s[i] = 0.f;
 #pragma unroll
-        for (int ks = 0; ks < C::KSTEPS; ks++) {
-            T8 a = as_vec<T8>(lds_read16(k_lds + SW::off(nh + r, ks * 16 + 8 * g)));
-            s = mfma32(a, qreg[ks], s);
+            for (int ks = 0; ks < C::KSTEPS; ks++) {
+                T8 a = as_vec<T8>(lds_read16(k_lds + SW::off(nh + r, ks * 16 + 8 * g)));
+                s = mfma32(a, qreg[ks], s);
+            }
+            if (nb == 0) ks_.template issue_ahead<BV>(k);  // in the shadow of the MFMAs just issued
         }
-        if (nb == 0) ks_.template issue_ahead<BV>(k);  // in the shadow of the MFMAs just issued
 
         // ---- online softmax step.  `masked` steps (ragged edge, causal diagonal) and a
         // non-positive scale follow the reference's arithmetic term by term: scaled score,

@@ -317,6 +317,27 @@ def test_bias_layouts(gpu_device):
             check(ours, ref, "%s %s causal=%s" % (name, dtype, causal))
 
 
+def test_seeded_random_shapes(gpu_device):
+    """A seeded sweep over head dims, dtypes, bias kinds, causal and shapes around every tile and
+    ring boundary (32, 64, 128, 256 and their neighbours, up to a few dozen steps)."""
+    import random
+    rnd = random.Random(20240)
+    sizes = [1, 7, 31, 32, 33, 64, 100, 128, 129, 200, 255, 256, 257, 384, 500, 640, 1100]
+    keys = [1, 8, 16, 31, 32, 33, 64, 77, 96, 128, 136, 200, 256, 264, 328, 512, 520, 1000, 1544]
+    for case in range(60):
+        D = rnd.choice([16, 32, 64, 64, 128, 128, 128, 256])
+        dtype = rnd.choice([torch.bfloat16, torch.float16])
+        causal = rnd.random() < 0.4
+        M = rnd.choice(sizes)
+        N = M if causal else rnd.choice(keys)
+        B, H = rnd.choice([(1, 1), (1, 2), (2, 3)])
+        kind = rnd.choice([None, "bool", "bf16", "f16", "bf16", "f32"])
+        trainable = rnd.random() < 0.7
+        q, k, v, do, bias = make_inputs(gpu_device, B, M, N, H, D, dtype, kind, seed=1000 + case, trainable=trainable)
+        check(run_ours(q, k, v, do, bias, causal), run_oracle(q, k, v, do, bias, causal),
+              "case %d D%d %s causal=%s %s bias=%s trainable=%s" % (case, D, dtype, causal, (B, M, N, H), kind, trainable))
+
+
 def test_repeatability(gpu_device):
     q, k, v, do, bias = make_inputs(gpu_device, 1, 512, 512, 4, 128, torch.bfloat16, "bf16", seed=33)
     a = run_ours(q, k, v, do, bias, False)

@@ -309,10 +309,11 @@ template <int D, int BIAS> struct BwdCfg {
     static constexpr int BCH = (BMI * BCPR + 63) / 64;     // bias copies per S-wave per block
     static constexpr int Q_BYTES = BMI * D * 2;
     static constexpr int NQD = Q_BYTES / 1024;             // 1 KB copies per Q (or dO) block
-    static constexpr int QD = NQD >= 4 ? NQD / 4 : 1;      // of which each S-wave issues this many
-    // Q, dO, LSE, delta and the bias slices reach LDS through direct global -> LDS copies that the
-    // S-waves issue LA blocks ahead of their use; a copy has LA - 1 whole steps and the rest of
-    // its own to land before the barrier that publishes it.
+    static constexpr int QD = NQD >= 4 ? NQD / 4 : 1;      // of which each wave of a role issues this many
+    // Q, dO, LSE, delta and the bias slices reach LDS through direct global -> LDS copies issued
+    // LA blocks ahead of their use (Q, LSE and bias by the S-waves, dO and delta by the dP-waves);
+    // a copy has LA - 1 whole steps and the rest of its own to land before the barrier that
+    // publishes it.
     static constexpr int DS_BYTES = (BIAS == 2 || BIAS == 3) ? BN * DSS * 2 : 0;  // dS^T tiles (dBias)
     static constexpr int P_BYTES = 4 * NSUB * 64 * 64;     // P hand-off: 16 floats per lane per sub-block
     static constexpr int BT_BYTES = BMI * 32 * ES;         // bias slice of one S-wave
@@ -340,9 +341,9 @@ template <int D, int BIAS> struct BwdCfg {
 // Work split inside a work-group of 8 waves.  Waves 0-3 ("S-waves") and waves 4-7 ("dP-waves")
 // pair up on the four 32-key blocks of the tile (waves w and w + 4 run on the same SIMD):
 //   S-wave : S = Q K^T, P = 2^(S*scale + bias - LSE)  -> hands P to its partner through LDS,
-//            dV^T += dO^T P
-//            and the global -> LDS copies of the Q / dO / LSE / delta / bias blocks
-//   dP-wave: dP = dO V^T, dS = P (dP - delta) (+ dBias through an LDS tile), dK^T += Q^T dS
+//            dV^T += dO^T P, and the global -> LDS copies of the Q / LSE / bias blocks
+//   dP-wave: dP = dO V^T, dS = P (dP - delta) (+ dBias through an LDS tile), dK^T += Q^T dS,
+//            and the global -> LDS copies of the dO / delta blocks
 // The roles are skewed by one query block so that a step needs a single barrier and nothing a
 // wave does inside a step depends on what its partner does in the same step:
 //   step t : S-wave : P(t+1) from Q(t+1), then dV += dO(t)^T P(t)        (P(t) kept in registers)
@@ -431,10 +432,10 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
         }
     }
 
-    // ---- global -> LDS copies of Q (+LSE), dO (+delta) and bias blocks, issued by the S-waves ----
+    // ---- global -> LDS copies of Q (+LSE), dO (+delta) and bias blocks ----
     // A block is NQD copies of 1 KB; copy ci fills bytes [1024 ci, 1024 ci + 1024) of the swizzled
     // tile, so lane l of it fetches the 16-byte chunk that lives at tile position 64 ci + l.  Each
-    // S-wave issues QD of them (more than once where a block has fewer than four), every step the
+    // wave of the issuing role issues QD of them (more than once where a block has fewer than four), every step the
     // same number: completion is counted (s_waitcnt vmcnt) and copies complete in issue order.
     // Rows past M re-read the last row: their P and dS are exactly zero.
     unsigned cq_off[C::QD], cdo_off[C::QD];

@@ -209,14 +209,25 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_
 #pragma unroll
                     for (int i = 0; i < 16; i++) o_acc[db][i] *= alpha;
             }
+            // ---- P and O^T += V^T P^T (A = V^T gathered down the columns of the V rows), 16 keys
+            // at a time: the MFMAs of the first 16 keys run while the exponentials of the second 16
+            // are computed ----
             float rs = 0.f;
 #pragma unroll
-            for (int i = 0; i < 16; i++) {
-                float pv;
-                if constexpr (RAW || NAT) pv = fast_exp2(__builtin_fmaf(s[i], to_log2, -m_i));
-                else pv = fast_exp2(s[i] - m_i);
-                rs += pv;
-                pb[i >> 3][i & 7] = (T)pv;
+            for (int kk = 0; kk < 2; kk++) {
+#pragma unroll
+                for (int i = kk * 8; i < kk * 8 + 8; i++) {
+                    float pv;
+                    if constexpr (RAW || NAT) pv = fast_exp2(__builtin_fmaf(s[i], to_log2, -m_i));
+                    else pv = fast_exp2(s[i] - m_i);
+                    rs += pv;
+                    pb[kk][i & 7] = (T)pv;
+                }
+#pragma unroll
+                for (int db = 0; db < C::DB; db++) {
+                    T8 a = SW::template col8<T8>(v_lds, lane, nh + kk * 16, db * 32);
+                    o_acc[db] = mfma32(a, pb[kk], o_acc[db]);
+                }
             }
             l_i += rs;  // per-lane partial sum; the two halves of a row are added at the end
         };
@@ -225,16 +236,6 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_
             else softmax_step(std::false_type{});
         } else {
             softmax_step(std::false_type{});
-        }
-
-        // ---- O^T += V^T P^T : A = V^T gathered down the columns of the V rows ----
-#pragma unroll
-        for (int kk = 0; kk < 2; kk++) {
-#pragma unroll
-            for (int db = 0; db < C::DB; db++) {
-                T8 a = SW::template col8<T8>(v_lds, lane, nh + kk * 16, db * 32);
-                o_acc[db] = mfma32(a, pb[kk], o_acc[db]);
-            }
         }
         }
     };

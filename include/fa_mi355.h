@@ -114,7 +114,7 @@ enum fa_bwd_stage {
 /* Enqueue only the selected stages of the backward (same arguments and checks as fa_bwd).
  * No counterpart in the reference: it exists so that a benchmark or profiler can bracket one
  * stage with events; FA_STAGE_MAIN and FA_STAGE_DQ both need the delta of FA_STAGE_PREP, and when
- * dbias is requested in the element type of q, FA_STAGE_DQ reads the dbias that FA_STAGE_MAIN
+ * dbias is requested in fp32 or in the element type of q, FA_STAGE_DQ reads the dbias that FA_STAGE_MAIN
  * wrote (it is the dS of the dQ product) and must run after it. */
 int fa_bwd_stages(const fa_bwd_args *args, void *stream, int stages);
 

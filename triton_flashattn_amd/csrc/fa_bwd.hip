@@ -50,13 +50,14 @@ __global__ __launch_bounds__(256) void fa_bwd_prep_kernel(const BwdParams p) {
 // (flash_attention.py:458-646).
 //
 // FROM_DS: when the key-tile kernel has just written dBias in the element type of q, that tensor IS
-// dS rounded exactly as the reference rounds it before this product (flash_attention.py:516-520).
-// The kernel then reads the dBias slices through the bias ring instead of the bias, skips both
-// recomputed products, the exponentials and the V rows, and is one product instead of three.
+// dS rounded exactly as the reference rounds it before this product (flash_attention.py:516-520);
+// an fp32 dBias is dS itself and is rounded here.  The kernel then reads the dBias slices through
+// the bias ring instead of the bias, skips both recomputed products, the exponentials and the V
+// rows, and is one product instead of three.
 template <typename T, int D, int BIAS, bool CAUSAL, bool FROM_DS = false>
 __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_dq_kernel(const BwdParams p) {
-    static_assert(!FROM_DS || (BIAS == 2 && __is_same(T, _Float16)) || (BIAS == 3 && __is_same(T, __bf16)),
-                  "dS can stand in for the recomputation only in the element type of q");
+    static_assert(!FROM_DS || BIAS == 4 || (BIAS == 2 && __is_same(T, _Float16)) || (BIAS == 3 && __is_same(T, __bf16)),
+                  "dS can stand in for the recomputation only in fp32 or in the element type of q");
     typedef StreamCfg<D, BIAS> C;
     typedef Swz<D> SW;
     typedef typename VecOf<T>::v8 T8;
@@ -153,7 +154,14 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_
 #pragma unroll
                 for (int q4 = 0; q4 < 4; q4++) {
                     const int nl = 8 * q4 + 4 * g;
-                    T4 hv = *reinterpret_cast<const T4*>(b_lds + ks_.b_off(r, nl));
+                    T4 hv;
+                    if constexpr (BIAS == 4) {
+                        const f32x4 w = *reinterpret_cast<const f32x4*>(b_lds + ks_.b_off(r, nl));
+#pragma unroll
+                        for (int e = 0; e < 4; e++) hv[e] = (T)w[e];
+                    } else {
+                        hv = *reinterpret_cast<const T4*>(b_lds + ks_.b_off(r, nl));
+                    }
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
                         const int i = q4 * 4 + e;
@@ -843,12 +851,17 @@ template <typename T, int D> static hipError_t launch_all(const BwdParams& p, in
     }
     if (stages & 4) {
         dim3 qgrid((unsigned)(p.n_mtiles * p.B * p.H));
-        // dBias in the element type of q, written a moment ago by the key-tile kernel in rows of whole
-        // 16-byte chunks, is the dS the dQ product needs
+        // dBias in fp32 or in the element type of q, written a moment ago by the key-tile kernel in
+        // rows of whole 16-byte chunks, is the dS the dQ product needs
         constexpr int DS_BIAS = __is_same(T, _Float16) ? 2 : 3;
         if (dbias && bias == DS_BIAS && p.dbias_vec) {
             if (causal) hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, DS_BIAS, true, true>), qgrid, dim3(256), 0, st, p);
             else hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, DS_BIAS, false, true>), qgrid, dim3(256), 0, st, p);
+            return hipGetLastError();
+        }
+        if (dbias && bias == 4 && p.dbias_vec) {
+            if (causal) hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, 4, true, true>), qgrid, dim3(256), 0, st, p);
+            else hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, 4, false, true>), qgrid, dim3(256), 0, st, p);
             return hipGetLastError();
         }
 #define FA_CASE(BK)                                                                                               \

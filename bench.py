@@ -118,7 +118,7 @@ def time_stages(cfg, iters):
     t_bwd = event_time_ms(lambda: run(_native.FA_STAGE_ALL), iters)
     run(_native.FA_STAGE_PREP)
     t_main = event_time_ms(lambda: run(_native.FA_STAGE_MAIN), iters)
-    t_dq = event_time_ms(lambda: run(_native.FA_STAGE_DQ), iters)
+    t_dq = event_time_ms(lambda: run(_native.FA_STAGE_DQ | _native.FA_STAGE_DQ_FROM_DBIAS), iters)
     return t_fwd, t_bwd, t_main, t_dq
 
 

@@ -108,14 +108,20 @@ enum fa_bwd_stage {
     FA_STAGE_PREP = 1, /* delta = rowsum(o * do)          (flash_attention.py:197-233) */
     FA_STAGE_MAIN = 2, /* dK, dV, dBias over key tiles    (flash_attention.py:237-454) */
     FA_STAGE_DQ = 4,   /* dQ over query tiles              (flash_attention.py:458-646) */
-    FA_STAGE_ALL = 7
+    FA_STAGE_ALL = 7,
+    /* modifier of FA_STAGE_DQ when it is enqueued WITHOUT FA_STAGE_MAIN in the same call: the
+     * caller vouches that args->dbias still holds what FA_STAGE_MAIN wrote for these very
+     * arguments, so that dQ may be formed from it (one matrix product instead of three) */
+    FA_STAGE_DQ_FROM_DBIAS = 8
 };
 
 /* Enqueue only the selected stages of the backward (same arguments and checks as fa_bwd).
  * No counterpart in the reference: it exists so that a benchmark or profiler can bracket one
- * stage with events; FA_STAGE_MAIN and FA_STAGE_DQ both need the delta of FA_STAGE_PREP, and when
- * dbias is requested in fp32 or in the element type of q, FA_STAGE_DQ reads the dbias that FA_STAGE_MAIN
- * wrote (it is the dS of the dQ product) and must run after it. */
+ * stage with events.  FA_STAGE_MAIN and FA_STAGE_DQ both need the delta of FA_STAGE_PREP.  When
+ * FA_STAGE_MAIN and FA_STAGE_DQ run in one call and dbias is requested in fp32 or in the element
+ * type of q, dQ is formed from the dbias just written (it is the dS of the dQ product); a call with
+ * FA_STAGE_DQ alone recomputes dS from q, k, v and the bias and never reads dbias, unless
+ * FA_STAGE_DQ_FROM_DBIAS is added.  Both routes agree within the rounding of dS to 16 bits. */
 int fa_bwd_stages(const fa_bwd_args *args, void *stream, int stages);
 
 #ifdef __cplusplus

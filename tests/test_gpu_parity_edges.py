@@ -1,0 +1,172 @@
+"""GPU parity tests of the corners: the saved LSE, fully masked rows (whose softmax runs over
+scores quantised by the additive -1.0e6 term), non-positive scales, and the backward stages run
+one by one.  Same tolerances as test_gpu_parity.py."""
+import pytest
+import torch
+
+import triton_flashattn_amd.flash_attention as fa_mod
+from triton_flashattn_amd import _native
+from triton_flashattn_amd.flash_attention import _flash_attn_fwd
+from oracle.attention_oracle import LN2, attention_forward, attention_forward_streamed
+from test_gpu_parity import GRAD_RTOL, OUT_ATOL, check, make_inputs, rel_l2, run_oracle, run_ours
+
+pytestmark = pytest.mark.gpu
+
+
+# ---------------------------------------------------------------- LSE (flash_attention.py:188-193)
+@pytest.mark.parametrize("D", [64, 128])
+def test_lse_matches_oracle_causal_bool_ragged(gpu_device, D):
+    """lse = m + log2(l) in log2 units, (B, H, M).  The kernel only raises its running maximum
+    when a block exceeds it by 2^8, so m + log2(l) is checked where that laziness could show:
+    causal rows of every length, bool masks, float biases, ragged edges."""
+    cases = [  # M, N, bias kind, causal, sm_scale
+        (300, 300, None, True, None), (257, 257, "bool", True, None), (200, 333, "bool", False, None),
+        (129, 500, "bf16", False, 0.3), (513, 513, "f32", True, None), (100, 77, "f16", False, 1.0),
+    ]
+    for i, (M, N, kind, causal, scale) in enumerate(cases):
+        dtype = torch.bfloat16 if i % 2 else torch.float16
+        q, k, v, do, bias = make_inputs(gpu_device, 2, M, N, 2, D, dtype, kind, seed=40 + i, trainable=False)
+        sm_scale = D ** -0.5 if scale is None else scale
+        # large scores in a few rows: the running maximum must move by far more than 2^8
+        q[:, 5] *= 30.0
+        o, lse = _flash_attn_fwd(q, k, v, bias, causal, sm_scale)
+        ref_o, ref_lse = attention_forward(q, k, v, bias, causal, sm_scale)
+        assert lse.shape == ref_lse.shape
+        assert torch.allclose(lse, ref_lse, atol=3e-3, rtol=1e-5), (M, N, kind, causal, (lse - ref_lse).abs().max())
+        assert (o.float() - ref_o).abs().max().item() <= OUT_ATOL
+
+
+# ---------------------------------------------------------------- fully masked rows
+def _quantisation_case(dev, M, N, dead_rows, dtype):
+    """Scores 0 and 0.03 (log2 units, sm_scale = ln 2) on alternating keys, values +8 / -8.  With
+    every key of a row masked the reference adds -1.0e6 to all of them (flash_attention.py:48-53):
+    fp32 then holds the scores in steps of 2^-4, both kinds of key round to the same value and the
+    row's output is 0; a softmax over the unquantised scores gives -0.083."""
+    D, H = 16, 1
+    q = torch.zeros(1, M, H, D, dtype=dtype, device=dev)
+    k = torch.zeros(1, N, H, D, dtype=dtype, device=dev)
+    v = torch.zeros(1, N, H, D, dtype=dtype, device=dev)
+    q[..., 0] = 1.0
+    k[:, 1::2, :, 0] = 0.03
+    v[:, 0::2] = 8.0
+    v[:, 1::2] = -8.0
+    mask = torch.ones(1, H, M, N, dtype=torch.bool, device=dev)
+    mask[:, :, dead_rows, :] = False
+    return q, k, v, mask
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_fully_masked_rows_see_quantised_scores(gpu_device, dtype):
+    M, N = 200, 328                      # interior key steps and a ragged last one; rows in four waves
+    dead = [3, 40, 77, 127, 128, 199]
+    q, k, v, mask = _quantisation_case(gpu_device, M, N, dead, dtype)
+    out, lse = _flash_attn_fwd(q, k, v, mask, False, LN2)
+    ref, ref_lse = attention_forward(q, k, v, mask, False, LN2)
+    unq, _ = attention_forward(q, k, v, None, False, LN2)   # what an unquantised softmax would give
+    live = [i for i in range(M) if i not in dead]
+    # the case separates the two behaviours by far more than the tolerance ...
+    assert (ref[:, dead] - unq[:, dead]).abs().max().item() > 5e-2
+    assert ref[:, dead].abs().max().item() < 1e-3
+    # ... and the kernel is on the reference's side of it, tightly
+    assert (out[:, dead].float() - ref[:, dead]).abs().max().item() < 5e-3
+    assert (out[:, live].float() - ref[:, live]).abs().max().item() < OUT_ATOL
+    assert torch.allclose(lse[..., dead], ref_lse[..., dead], atol=0.07)  # one fp32 step at 1e6
+    assert torch.allclose(lse[..., live], ref_lse[..., live], atol=3e-3)
+
+
+def test_fully_masked_rows_causal_follow_a_reference_schedule(gpu_device):
+    """Causal + bool mask with rows whose visible keys are all masked.  Which causally hidden keys
+    such a row still sees depends on the reference's row-tile height (flash_attention.py:156-185), so the result
+    must be finite and equal to the streamed restatement for one of its tile heights."""
+    B, S, H, D = 1, 300, 2, 64
+    q, k, v, do, _ = make_inputs(gpu_device, B, S, S, H, D, torch.bfloat16, None, seed=51)
+    mask = torch.rand(B, H, S, S, device=gpu_device) > 0.3
+    mask[..., 0] = True
+    dead = [0, 5, 33, 64, 130, 299]
+    for r in dead:
+        mask[:, :, r, : r + 1] = False
+    ours = run_ours(q, k, v, do, mask, True)
+    for n in ("out", "dq", "dk", "dv"):
+        assert torch.isfinite(ours[n].float()).all(), n
+    o, lse = _flash_attn_fwd(q, k, v, mask, True, D ** -0.5)
+    assert torch.isfinite(lse).all()
+    errs = {}
+    for bm in (32, 64, 128):
+        ref, ref_lse = attention_forward_streamed(q, k, v, mask, True, None, block_m=bm, block_n=32)
+        errs[bm] = (o.float() - ref).abs().max().item()
+    assert min(errs.values()) <= OUT_ATOL, errs
+    # rows with a visible key do not depend on the schedule at all
+    live = [i for i in range(S) if i not in dead]
+    ref, _ = attention_forward(q, k, v, mask, True)
+    assert (o[:, live].float() - ref[:, live]).abs().max().item() <= OUT_ATOL
+
+
+# ---------------------------------------------------------------- non-positive scales
+@pytest.mark.parametrize("sm_scale", [-0.1, 0.0])
+@pytest.mark.parametrize("bias_kind", [None, "bool", "bf16"])
+def test_nonpositive_scale(gpu_device, sm_scale, bias_kind):
+    """With sm_scale <= 0 the largest raw score is no longer the largest scaled one: the kernels
+    must not fold the scale into a maximum taken over raw scores."""
+    for causal, (M, N) in ((False, (150, 200)), (True, (257, 257))):
+        q, k, v, do, bias = make_inputs(gpu_device, 1, M, N, 2, 64, torch.bfloat16, bias_kind, seed=60)
+        ours = run_ours(q, k, v, do, bias, causal, sm_scale)
+        ref = run_oracle(q, k, v, do, bias, causal, sm_scale)
+        check(ours, ref, "scale %g %s causal=%s" % (sm_scale, bias_kind, causal))
+        o, lse = _flash_attn_fwd(q, k, v, None if bias is None else bias.detach(), causal, sm_scale)
+        assert torch.allclose(lse, ref["lse2"], atol=3e-3, rtol=1e-5)
+
+
+# ---------------------------------------------------------------- backward stages
+def _stage_inputs(dev, bias_dtype, N=328):
+    B, M, H, D = 2, 200, 2, 128
+    g = torch.Generator(device="cpu").manual_seed(70)
+    mk = lambda *s: torch.randn(*s, generator=g).bfloat16().to(dev)
+    q, k, v, do = mk(B, M, H, D), mk(B, N, H, D), mk(B, N, H, D), mk(B, M, H, D)
+    bias = torch.randn(B, H, M, N, generator=g).to(bias_dtype).to(dev)
+    o, lse = _flash_attn_fwd(q, k, v, bias, False, D ** -0.5)
+    return q, k, v, do, bias, o, lse, D ** -0.5
+
+
+def _run_stages(args, stage_list, dbias_like=None, poison_dbias_before=None):
+    q, k, v, do, bias, o, lse, scale = args
+    dq, dk, dv = torch.full_like(q, 7.0), torch.full_like(k, 7.0), torch.full_like(v, 7.0)
+    dbias = torch.full_like(bias, 7.0) if dbias_like is None else dbias_like
+    ws = fa_mod._backend.bwd_workspace(q, k, bias, False, scale)
+    for st in stage_list:
+        if poison_dbias_before == st:
+            dbias.fill_(float("nan"))
+        fa_mod._backend.bwd(do, q, k, v, o, bias, False, scale, lse, dq, dk, dv, dbias, stages=st, workspace=ws)
+    torch.cuda.synchronize()
+    return dq, dk, dv, dbias
+
+
+@pytest.mark.parametrize("bias_dtype", [torch.bfloat16, torch.float32])
+def test_stages_one_by_one_equal_one_call(gpu_device, bias_dtype):
+    S = _native
+    args = _stage_inputs(gpu_device, bias_dtype)
+    whole = _run_stages(args, [S.FA_STAGE_ALL])
+    split = _run_stages(args, [S.FA_STAGE_PREP, S.FA_STAGE_MAIN, S.FA_STAGE_DQ | S.FA_STAGE_DQ_FROM_DBIAS])
+    for name, a, b in zip(("dq", "dk", "dv", "dbias"), whole, split):
+        assert torch.equal(a, b), name
+    # FA_STAGE_DQ alone recomputes dS: it never reads dbias (poisoned here) and agrees with the
+    # one-product route within the rounding of dS
+    alone = _run_stages(args, [S.FA_STAGE_PREP, S.FA_STAGE_MAIN, S.FA_STAGE_DQ], poison_dbias_before=S.FA_STAGE_DQ)
+    assert torch.isfinite(alone[0].float()).all()
+    assert rel_l2(alone[0], whole[0].float()) < 1e-2
+    assert torch.equal(alone[1], whole[1]) and torch.equal(alone[2], whole[2])
+
+
+def test_dq_routes_agree(gpu_device):
+    """dQ from the dBias just written (one product) against dQ recomputed from q, k, v and the bias
+    (three products; taken when dBias rows are not whole 16-byte chunks, here N = 324... odd rows)."""
+    args_fast = _stage_inputs(gpu_device, torch.bfloat16, N=328)
+    whole = _run_stages(args_fast, [_native.FA_STAGE_ALL])
+    # the same problem with a dBias whose rows are padded to an odd stride: the dispatcher cannot
+    # use 16-byte stores, writes dBias element by element and recomputes dS in the dQ kernel
+    q, k, v, do, bias, o, lse, scale = args_fast
+    padded = torch.full((2, 2, 200, 329), 7.0, dtype=bias.dtype, device=bias.device)[..., :328]
+    slow = _run_stages(args_fast, [_native.FA_STAGE_ALL], dbias_like=padded)
+    assert rel_l2(slow[0], whole[0].float()) < 1e-2
+    assert rel_l2(slow[3], whole[3].float()) < 1e-3
+    for i in (1, 2):
+        assert rel_l2(slow[i], whole[i].float()) < 1e-2

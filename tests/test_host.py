@@ -218,3 +218,6 @@ def test_abi_status_codes_and_workspace():
     assert lib.fa_bwd(ctypes.byref(b), None) == -6            # no workspace
     b.dbias = base
     assert lib.fa_bwd(ctypes.byref(b), None) == -4            # dbias without a float bias
+    b.dbias = None
+    assert lib.fa_bwd_stages(ctypes.byref(b), None, 16) == -7                       # unknown stage bit
+    assert lib.fa_bwd_stages(ctypes.byref(b), None, _native.FA_STAGE_DQ_FROM_DBIAS) == -7   # modifier alone

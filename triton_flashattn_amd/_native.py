@@ -6,8 +6,7 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-# FA_MI355_LIB points at another build of the same ABI (e.g. an instrumented one)
-LIB_PATH = os.environ.get("FA_MI355_LIB") or os.path.join(_HERE, "libfa_mi355.so")
+LIB_PATH = os.path.join(_HERE, "libfa_mi355.so")
 ABI_VERSION = 1
 
 FA_F16, FA_BF16 = 0, 1
@@ -48,7 +47,7 @@ class FaBwdArgs(ctypes.Structure):
 
 
 EXPORTS = ("fa_abi_version", "fa_strerror", "fa_fwd", "fa_bwd_workspace_bytes", "fa_bwd", "fa_bwd_stages")
-FA_STAGE_PREP, FA_STAGE_MAIN, FA_STAGE_DQ, FA_STAGE_ALL = 1, 2, 4, 7
+FA_STAGE_PREP, FA_STAGE_MAIN, FA_STAGE_DQ, FA_STAGE_ALL, FA_STAGE_DQ_FROM_DBIAS = 1, 2, 4, 7, 8
 
 _lib = None
 

@@ -11,7 +11,9 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libfa_mi355.so")
-SOURCES = ["fa_fwd.hip", "fa_bwd.hip", "fa_api.hip"]
+HEAD_DIMS = (128, 64, 256, 32, 16)  # longest compiles first
+# (source, head dim or None): the kernel files are compiled once per head dimension
+UNITS = [("fa_bwd.hip", d) for d in HEAD_DIMS] + [("fa_fwd.hip", d) for d in HEAD_DIMS] + [("fa_api.hip", None)]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-munsafe-fp-atomics",
@@ -21,19 +23,21 @@ FLAGS = [
 ]
 
 
-def _compile(src):
-    obj = os.path.join(CSRC, src.replace(".hip", ".o"))
-    cmd = [HIPCC] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+def _compile(unit):
+    src, d = unit
+    obj = os.path.join(CSRC, src.replace(".hip", ".o" if d is None else "_d%d.o" % d))
+    defs = [] if d is None else ["-DFA_HEAD_DIM=%d" % d]
+    cmd = [HIPCC] + FLAGS + defs + ["-c", os.path.join(CSRC, src), "-o", obj]
     res = subprocess.run(cmd, capture_output=True, text=True)
     log = "\n".join(l for l in (res.stdout + res.stderr).splitlines() if "packed-fp32-ops" not in l)
     if res.returncode != 0:
-        raise RuntimeError("hipcc failed for %s:\n%s" % (src, log))
+        raise RuntimeError("hipcc failed for %s (D=%s):\n%s" % (src, d, log))
     return obj, log
 
 
-def build(jobs=4, verbose=False):
+def build(jobs=8, verbose=False):
     with ThreadPoolExecutor(max_workers=max(1, jobs)) as ex:
-        results = list(ex.map(_compile, SOURCES))
+        results = list(ex.map(_compile, UNITS))
     objs = [o for o, _ in results]
     if verbose:
         for _, log in results:
@@ -47,7 +51,7 @@ def build(jobs=4, verbose=False):
 
 
 if __name__ == "__main__":
-    j = 4
+    j = 8
     if "-j" in sys.argv:
         j = int(sys.argv[sys.argv.index("-j") + 1])
     print(build(jobs=j, verbose=True))

@@ -6,10 +6,42 @@
 #include "fa_params.hpp"
 
 namespace fa {
-hipError_t launch_fwd(const FwdParams& p, int D, int dtype, int bias, bool causal, hipStream_t st);
-hipError_t launch_bwd(const BwdParams& p, int D, int dtype, int bias, bool causal, bool dbias, int stages, hipStream_t st);
-int fwd_block_m();
-int bwd_block_n(int D);
+// one object file per head dimension defines these (fa_fwd.hip, fa_bwd.hip with -DFA_HEAD_DIM)
+template <int D> hipError_t launch_fwd_d(const FwdParams& p, int dtype, int bias, bool causal, hipStream_t st);
+template <int D> hipError_t launch_bwd_d(const BwdParams& p, int dtype, int bias, bool causal, bool dbias, int stages, hipStream_t st);
+#define FA_DECLARE_D(D)                                                                                         \
+    template <> hipError_t launch_fwd_d<D>(const FwdParams& p, int dtype, int bias, bool causal, hipStream_t st); \
+    template <> hipError_t launch_bwd_d<D>(const BwdParams& p, int dtype, int bias, bool causal, bool dbias, int stages, hipStream_t st);
+FA_DECLARE_D(16)
+FA_DECLARE_D(32)
+FA_DECLARE_D(64)
+FA_DECLARE_D(128)
+FA_DECLARE_D(256)
+#undef FA_DECLARE_D
+
+static hipError_t launch_fwd(const FwdParams& p, int D, int dtype, int bias, bool causal, hipStream_t st) {
+    switch (D) {
+        case 16: return launch_fwd_d<16>(p, dtype, bias, causal, st);
+        case 32: return launch_fwd_d<32>(p, dtype, bias, causal, st);
+        case 64: return launch_fwd_d<64>(p, dtype, bias, causal, st);
+        case 128: return launch_fwd_d<128>(p, dtype, bias, causal, st);
+        case 256: return launch_fwd_d<256>(p, dtype, bias, causal, st);
+    }
+    return hipErrorNotSupported;
+}
+static hipError_t launch_bwd(const BwdParams& p, int D, int dtype, int bias, bool causal, bool dbias, int stages, hipStream_t st) {
+    switch (D) {
+        case 16: return launch_bwd_d<16>(p, dtype, bias, causal, dbias, stages, st);
+        case 32: return launch_bwd_d<32>(p, dtype, bias, causal, dbias, stages, st);
+        case 64: return launch_bwd_d<64>(p, dtype, bias, causal, dbias, stages, st);
+        case 128: return launch_bwd_d<128>(p, dtype, bias, causal, dbias, stages, st);
+        case 256: return launch_bwd_d<256>(p, dtype, bias, causal, dbias, stages, st);
+    }
+    return hipErrorNotSupported;
+}
+// query rows per work-group of the forward and dQ kernels; keys per work-group of the dK/dV kernel
+static int fwd_block_m() { return 128; }
+static int bwd_block_n(int) { return 128; }
 }  // namespace fa
 
 namespace {
@@ -125,9 +157,15 @@ size_t fa_bwd_workspace_bytes(const fa_problem* p) {
     return align256(rows * sizeof(float));
 }
 
-int fa_bwd_stages(const fa_bwd_args* a, void* stream, int stages) {
+}  // extern "C"
+
+namespace {
+
+// `delta` NULL: the scratch is the caller's workspace; else the workspace fields are ignored
+int bwd_enqueue(const fa_bwd_args* a, void* stream, int stages, float* delta) {
     if (!a) return FA_ERR_NULL;
-    if (stages <= 0 || (stages & ~FA_STAGE_ALL)) return FA_ERR_UNSUPPORTED;
+    if (stages <= 0 || (stages & ~(FA_STAGE_ALL | FA_STAGE_DQ_FROM_DBIAS))) return FA_ERR_UNSUPPORTED;
+    if ((stages & FA_STAGE_DQ_FROM_DBIAS) && !(stages & FA_STAGE_DQ)) return FA_ERR_UNSUPPORTED;
     const fa_problem& p = a->p;
     int st = check_problem(p);
     if (st != FA_OK) return st;
@@ -139,14 +177,17 @@ int fa_bwd_stages(const fa_bwd_args* a, void* stream, int stages) {
         !qkv_layout_ok(a->dout, a->do_strides, p.B, p.M, p.H) || !qkv_layout_ok(a->dq, a->dq_strides, p.B, p.M, p.H) ||
         !qkv_layout_ok(a->dk, a->dk_strides, p.B, p.N, p.H) || !qkv_layout_ok(a->dv, a->dv_strides, p.B, p.N, p.H))
         return FA_ERR_LAYOUT;
-    size_t need = fa_bwd_workspace_bytes(&p);
-    if (!a->workspace || a->workspace_bytes < need || reinterpret_cast<uintptr_t>(a->workspace) % 256 != 0)
-        return FA_ERR_WORKSPACE;
+    if (!delta) {
+        size_t need = fa_bwd_workspace_bytes(&p);
+        if (!a->workspace || a->workspace_bytes < need || reinterpret_cast<uintptr_t>(a->workspace) % 256 != 0)
+            return FA_ERR_WORKSPACE;
+        delta = static_cast<float*>(a->workspace);
+    }
 
     fa::BwdParams k{};
     k.q = a->q; k.k = a->k; k.v = a->v; k.o = a->o; k.dout = a->dout; k.bias = a->bias; k.lse = a->lse;
     k.dq = a->dq; k.dk = a->dk; k.dv = a->dv; k.dbias = a->dbias;
-    k.delta = static_cast<float*>(a->workspace);
+    k.delta = delta;
     k.sq = s3(a->q_strides); k.sk = s3(a->k_strides); k.sv = s3(a->v_strides); k.so = s3(a->o_strides);
     k.sdo = s3(a->do_strides); k.sdq = s3(a->dq_strides); k.sdk = s3(a->dk_strides); k.sdv = s3(a->dv_strides);
     if (a->bias) {
@@ -169,6 +210,12 @@ int fa_bwd_stages(const fa_bwd_args* a, void* stream, int stages) {
     return e == hipSuccess ? FA_OK : FA_ERR_LAUNCH;
 }
 
-int fa_bwd(const fa_bwd_args* a, void* stream) { return fa_bwd_stages(a, stream, FA_STAGE_ALL); }
+}  // namespace
+
+extern "C" {
+
+int fa_bwd_stages(const fa_bwd_args* a, void* stream, int stages) { return bwd_enqueue(a, stream, stages, nullptr); }
+
+int fa_bwd(const fa_bwd_args* a, void* stream) { return bwd_enqueue(a, stream, FA_STAGE_ALL, nullptr); }
 
 }  // extern "C"

@@ -302,6 +302,46 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_
 
 
 // ---------------------------------------------------------------------------------------------
+// The bias of 4 consecutive query rows at one key, as the dK/dV kernel reads it from a row-major
+// slice (32 keys per row) in LDS; get(e) is the additive term of row e: natural units for a float
+// bias, log2 units (0 or the mask value) for a bool mask.
+template <int BIAS> struct BiasQuad;
+template <> struct BiasQuad<0> {
+    __device__ __forceinline__ void load(const unsigned char*, int, int, int) {}
+    __device__ __forceinline__ float get(int) const { return 0.f; }
+};
+template <> struct BiasQuad<1> {
+    unsigned char v[4];
+    __device__ __forceinline__ void load(const unsigned char* slice, int row0, int key, int) {
+#pragma unroll
+        for (int e = 0; e < 4; e++) v[e] = slice[(row0 + e) * 32 + key];
+    }
+    __device__ __forceinline__ float get(int e) const { return v[e] ? 0.f : kMask; }
+};
+template <> struct BiasQuad<2> {
+    i16x4 raw;  // 4 rows of one key column in one transposing read
+    __device__ __forceinline__ void load(const unsigned char* slice, int row0, int, int lane) {
+        raw = lds_read_tr4(reinterpret_cast<const _Float16*>(slice) + tr_offset(lane, row0, 0, 32));
+    }
+    __device__ __forceinline__ float get(int e) const { return (float)__builtin_bit_cast(f16x4, raw)[e]; }
+};
+template <> struct BiasQuad<3> {
+    i16x4 raw;
+    __device__ __forceinline__ void load(const unsigned char* slice, int row0, int, int lane) {
+        raw = lds_read_tr4(reinterpret_cast<const __bf16*>(slice) + tr_offset(lane, row0, 0, 32));
+    }
+    __device__ __forceinline__ float get(int e) const { return (float)__builtin_bit_cast(bf16x4, raw)[e]; }
+};
+template <> struct BiasQuad<4> {
+    float v[4];
+    __device__ __forceinline__ void load(const unsigned char* slice, int row0, int key, int) {
+#pragma unroll
+        for (int e = 0; e < 4; e++) v[e] = reinterpret_cast<const float*>(slice)[(row0 + e) * 32 + key];
+    }
+    __device__ __forceinline__ float get(int e) const { return v[e]; }
+};
+
+// ---------------------------------------------------------------------------------------------
 template <int D, int BIAS> struct BwdCfg {
     static constexpr int BN = 128, NT = 512;
     static constexpr int NSUB = (D <= 64 && BIAS == 0) ? 2 : 1;  // 32-row sub-blocks of a query block
@@ -550,45 +590,82 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
 #pragma unroll
         for (int kk = 0; kk < 2; kk++) op_cur[sb][kk] = as_vec<T8>(i32x4{0, 0, 0, 0});
 
+    // A wave issues its instructions in order and only two waves share a SIMD, so every LDS round
+    // trip that sits between two dependent pieces of a step is dead time.  A step therefore
+    // fetches what it needs from LDS into registers at its top (PRELOAD): the A operands of both
+    // products and the inputs of the element-wise work, each ahead of work that hides the trip.
+    // With D = 256 there is no register room for that and the compiler places the reads.
+    constexpr bool PRELOAD = D <= 128;
+    constexpr int NR = NSUB * C::KSTEPS;  // A operands of a row product: 32 rows x 16 of the head dim each
+    constexpr int NA = NSUB * 2 * C::DB;  // A operands of a column product: 32 of the head dim x 16 rows each
+    // tiles are named by their LDS byte address (scalar); the two per-lane address constants of
+    // Swz cover every operand read of the loop
+    const unsigned rows_l = SW::rows_lane(lane), cols_l = SW::cols_lane(lane);
+    auto load_rows = [&](unsigned tile, T8 (&a)[NR]) {
+        const unsigned base = tile + rows_l;
+#pragma unroll
+        for (int sb = 0; sb < NSUB; sb++)
+#pragma unroll
+            for (int ks = 0; ks < C::KSTEPS; ks++) a[sb * C::KSTEPS + ks] = SW::template row8_at<T8>(base, sb * 32, ks);
+    };
     // sacc = rows(tile) x opreg: S = Q K^T (S-wave) or dP = dO V^T (dP-wave)
-    auto gemm_rows = [&](const T* tile, f32x16 (&sacc)[NSUB]) {
+    auto mma_rows = [&](const T8 (&a)[NR], f32x16 (&sacc)[NSUB]) {
 #pragma unroll
         for (int sb = 0; sb < NSUB; sb++) {
 #pragma unroll
             for (int i = 0; i < 16; i++) sacc[sb][i] = 0.f;
 #pragma unroll
-            for (int ks = 0; ks < C::KSTEPS; ks++) {
-                T8 a = as_vec<T8>(lds_read16(tile + SW::off(sb * 32 + r, ks * 16 + 8 * g)));
-                sacc[sb] = mfma32(a, opreg[ks], sacc[sb]);
-            }
+            for (int ks = 0; ks < C::KSTEPS; ks++) sacc[sb] = mfma32(a[sb * C::KSTEPS + ks], opreg[ks], sacc[sb]);
         }
     };
-    // acc^T += tile^T op: dV^T += dO^T P (S-wave) or dK^T += Q^T dS (dP-wave); the A operands are
-    // columns of the tile gathered with ds_read_b64_tr_b16
-    auto gemm_cols = [&](const T* tile, const T8 (&op)[NSUB][2]) {
+    // the A operands of acc^T += tile^T op are columns of the tile, gathered with ds_read_b64_tr_b16
+    auto load_cols = [&](unsigned tile, T8 (&a)[NA]) {
+        const unsigned base = tile + cols_l;
 #pragma unroll
         for (int sb = 0; sb < NSUB; sb++)
 #pragma unroll
             for (int kk = 0; kk < 2; kk++)
 #pragma unroll
-                for (int db = 0; db < C::DB; db++) {
-                    T8 a = SW::template col8<T8>(tile, lane, sb * 32 + kk * 16, db * 32);
-                    acc[db] = mfma32(a, op[sb][kk], acc[db]);
-                }
+                for (int db = 0; db < C::DB; db++)
+                    a[(sb * 2 + kk) * C::DB + db] = SW::template col8_at<T8>(base, sb * 32 + kk * 16, db);
     };
+    // acc^T += tile^T op: dV^T += dO^T P (S-wave) or dK^T += Q^T dS (dP-wave)
+    auto mma_cols = [&](const T8 (&a)[NA], const T8 (&op)[NSUB][2]) {
+#pragma unroll
+        for (int sb = 0; sb < NSUB; sb++)
+#pragma unroll
+            for (int kk = 0; kk < 2; kk++)
+#pragma unroll
+                for (int db = 0; db < C::DB; db++) acc[db] = mfma32(a[(sb * 2 + kk) * C::DB + db], op[sb][kk], acc[db]);
+    };
+    // ring slots of a block index that may run one or two blocks below zero at the first steps
+    auto q_tile = [&](int mb) { return lds_base + (unsigned)(((mb < 0 ? 0 : mb) % C::NQB) * C::Q_BYTES); };
+    auto do_tile = [&](int mb) { return lds_base + (unsigned)(C::OFF_DO + ((mb < 0 ? 0 : mb) % C::NDOB) * C::Q_BYTES); };
 
     if (s_wave) {
         // ================================ S-wave ================================
         auto s_loop = [&](auto bv_tag) {
         constexpr bool BV = decltype(bv_tag)::value;                    // bias slices come by copy
         constexpr int OPS = (BV ? C::BCH : 0) + ((Q_BY_S ? 1 : 0) + (DO_BY_S ? 1 : 0)) * (C::QD + 1);  // copies per step
-#pragma unroll 1
-        for (int t = mb_first - 1; t <= n_mblocks; t++) {
+        // S_AHEAD: the scores of a block are formed at the END of the step before the one that turns
+        // them into P, so that a step of this role opens with vector work (exponentials) while the
+        // partner wave on the same SIMD opens with matrix products, and closes with matrix products
+        // while the partner does its vector work.  It needs the Q block one step earlier, i.e. a copy
+        // look-ahead of at least three blocks.  Measured: 6 % on the kernel with a bias (where the
+        // vector work is heaviest), a loss of 4 % without one, which keeps the plain order.
+        constexpr bool S_AHEAD = BIAS != 0 && C::LA >= 3;
+        f32x16 sacc[NSUB];
+        if constexpr (S_AHEAD) {
+            T8 a_rows[NR];
+            load_rows(q_tile(mb_first), a_rows);
+            mma_rows(a_rows, sacc);
+        }
+        auto s_step = [&](int t) {
             const int nb = t + 1;  // the block whose P is produced in this step
             T8 op_next[NSUB][2];
             // Copies for the steps to come (their buffers were last read one step ago).  With a bias
-            // they are issued in the shadow of the first MFMAs of the step, without one right
-            // after the barrier: measured, each way is a few per cent better in its case.
+            // they are issued behind the LDS reads of the step, whose round trip they cover; without
+            // one right after the barrier: measured, each way is a few per cent better in its case.
             auto issue_copies = [&]() {
                 const unsigned saved_m0 = lds_copy_begin();
                 if constexpr (Q_BY_S) issue_q(nb + C::LA);
@@ -596,53 +673,43 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
                 if constexpr (DO_BY_S) issue_do(t + C::LA);
                 lds_copy_end(saved_m0);
             };
-            if constexpr (BIAS == 0) issue_copies();
-            // dV^T += dO(t)^T P(t) first: its operands are ready, and the Q rows of the next block
-            // can be on their way out of LDS meanwhile
-            if (t >= mb_first && t < n_mblocks)
-                gemm_cols(reinterpret_cast<const T*>(smem + C::OFF_DO + (t % C::NDOB) * C::Q_BYTES), op_cur);
-            if constexpr (BIAS != 0) issue_copies();
-            if (nb < n_mblocks) {
+            const unsigned char* bt_lds = ring_lds + ((nb - mb_first) % C::RING) * C::BT_BYTES;
+            const float* lse_lds = reinterpret_cast<const float*>(smem + C::OFF_LSE) + (nb % C::NQB) * BMI;
+            // inputs of P: LSE of 4 consecutive rows and the bias of those rows at this lane's key
+            f32x4 lse_in[NSUB][4];
+            BiasQuad<BIAS> bias_in[NSUB][4];
+            auto load_p_inputs = [&]() {
+#pragma unroll
+                for (int sb = 0; sb < NSUB; sb++)
+#pragma unroll
+                    for (int q4 = 0; q4 < 4; q4++) {
+                        const int ml0 = sb * 32 + 8 * q4 + 4 * g;  // first of 4 consecutive rows
+                        lse_in[sb][q4] = *reinterpret_cast<const f32x4*>(lse_lds + ml0);
+                        bias_in[sb][q4].load(bt_lds, ml0, r, lane);
+                    }
+            };
+            // ---- P (flash_attention.py:281-294) of block nb from its scores; register i of sub-block
+            // sb is row m0 + 32 sb + 8 (i/4) + 4 g + i%4, the lane is key my_n.  Blocks that touch a
+            // ragged edge or the causal diagonal follow the reference's additive -1e6 arithmetic term
+            // by term; interior blocks fold everything into one exponent. ----
+            auto make_p = [&]() {
                 const int m0 = nb * BMI;
-                const unsigned char* bt_lds = ring_lds + ((nb - mb_first) % C::RING) * C::BT_BYTES;
-                if constexpr (BIAS != 0 && !BV)
-                    load_bias_scalar(nb, ring_lds + ((nb - mb_first) % C::RING) * C::BT_BYTES);
                 const bool need_mask = (m0 + BMI > M) || (n0 + BN > N) || (CAUSAL && m0 < n0 + BN - 1);
-                f32x16 sacc[NSUB];
-                gemm_rows(reinterpret_cast<const T*>(smem + (nb % C::NQB) * C::Q_BYTES), sacc);
-                const float* lse_lds = reinterpret_cast<const float*>(smem + C::OFF_LSE) + (nb % C::NQB) * BMI;
                 float* p_out = p_lds + (nb & 1) * (C::P_BYTES / 4);
-                // ---- P (flash_attention.py:281-294); register i of sub-block sb is row
-                // m0 + 32 sb + 8 (i/4) + 4 g + i%4, the lane is key my_n.  Blocks that touch a ragged
-                // edge or the causal diagonal follow the reference's additive -1e6 arithmetic term by
-                // term; interior blocks fold everything into one exponent. ----
                 auto p_step = [&](auto masked_tag) {
                     constexpr bool MASKED = decltype(masked_tag)::value;
 #pragma unroll
                     for (int sb = 0; sb < NSUB; sb++) {
 #pragma unroll
                         for (int q4 = 0; q4 < 4; q4++) {
-                            const int ml0 = sb * 32 + 8 * q4 + 4 * g;  // first of 4 consecutive rows
-                            const f32x4 lse4 = *reinterpret_cast<const f32x4*>(lse_lds + ml0);
-                            // bool mask: the additive term in log2 units; float bias: natural units
-                            float bv[4] = {0.f, 0.f, 0.f, 0.f};
-                            if constexpr (BIAS == 1) {
-#pragma unroll
-                                for (int e = 0; e < 4; e++) bv[e] = bt_lds[(ml0 + e) * 32 + r] ? 0.f : kMask;
-                            } else if constexpr (BIAS == 2 || BIAS == 3) {
-                                typedef typename VecOf<E>::v4 B4;
-                                i16x4 raw = lds_read_tr4(reinterpret_cast<const E*>(bt_lds) + tr_offset(lane, ml0, 0, 32));
-                                B4 hv = __builtin_bit_cast(B4, raw);
-#pragma unroll
-                                for (int e = 0; e < 4; e++) bv[e] = (float)hv[e];
-                            } else if constexpr (BIAS == 4) {
-#pragma unroll
-                                for (int e = 0; e < 4; e++) bv[e] = reinterpret_cast<const float*>(bt_lds)[(ml0 + e) * 32 + r];
-                            }
+                            const int ml0 = sb * 32 + 8 * q4 + 4 * g;
+                            const f32x4 lse4 = lse_in[sb][q4];
                             f32x4 p4;
 #pragma unroll
                             for (int e = 0; e < 4; e++) {
                                 const int i = q4 * 4 + e;
+                                // bool mask: the additive term in log2 units; float bias: natural units
+                                const float bv = bias_in[sb][q4].get(e);
                                 float pv;
                                 if constexpr (MASKED) {
                                     const int m = m0 + ml0 + e;
@@ -650,12 +717,12 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
                                     const bool oob = (m >= M) || (my_n >= N);
                                     float tmask = oob ? kMask : 0.f;
                                     if (CAUSAL) tmask += (m < my_n) ? kMask : 0.f;
-                                    float add = BIAS >= 2 ? __fmul_rn(bv[e], kLog2e) : bv[e];
+                                    float add = BIAS >= 2 ? __fmul_rn(bv, kLog2e) : bv;
                                     if (BIAS != 0) add = oob ? kMask : add;
                                     x = __fadd_rn(x, __fadd_rn(tmask, add));
                                     pv = fast_exp2(x - lse4[e]);
                                 } else {
-                                    const float off = BIAS >= 2 ? __builtin_fmaf(bv[e], kLog2e, -lse4[e]) : bv[e] - lse4[e];
+                                    const float off = BIAS >= 2 ? __builtin_fmaf(bv, kLog2e, -lse4[e]) : bv - lse4[e];
                                     pv = fast_exp2(__builtin_fmaf(sacc[sb][i], qk_scale, off));
                                 }
                                 p4[e] = pv;
@@ -668,15 +735,59 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
                 };
                 if (need_mask) p_step(std::true_type{});
                 else p_step(std::false_type{});
+            };
+            if constexpr (BIAS != 0 && !BV) {
+                if (nb < n_mblocks) load_bias_scalar(nb, ring_lds + ((nb - mb_first) % C::RING) * C::BT_BYTES);
+            }
+            if constexpr (S_AHEAD) {
+                // vector work first: P(nb) from the scores formed at the end of the last step
+                T8 a_cols[NA], a_rows[NR];
+                if constexpr (PRELOAD) {
+                    load_p_inputs();
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                issue_copies();  // behind the reads, whose round trip they cover
+                if constexpr (!PRELOAD) load_p_inputs();
+                if (nb < n_mblocks) make_p();
+                if constexpr (PRELOAD) __builtin_amdgcn_sched_barrier(0);
+                load_cols(do_tile(t), a_cols);
+                load_rows(q_tile(nb + 1), a_rows);  // lands while the first product runs
+                if constexpr (PRELOAD) __builtin_amdgcn_sched_barrier(0);
+                // dV^T += dO(t)^T P(t), then the scores of block nb + 1 for the next step
+                if (t >= mb_first && t < n_mblocks) mma_cols(a_cols, op_cur);
+                if (nb + 1 < n_mblocks) mma_rows(a_rows, sacc);
+            } else {
+                T8 a_cols[NA], a_rows[NR];
+                if constexpr (BIAS == 0) issue_copies();
+                load_cols(do_tile(t), a_cols);
+                load_rows(q_tile(nb), a_rows);
+                if constexpr (PRELOAD) {
+                    load_p_inputs();
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                if constexpr (BIAS != 0) issue_copies();
+                // dV^T += dO(t)^T P(t) first: its operands do not depend on this step
+                if (t >= mb_first && t < n_mblocks) mma_cols(a_cols, op_cur);
+                if (nb < n_mblocks) {
+                    mma_rows(a_rows, sacc);
+                    if constexpr (!PRELOAD) load_p_inputs();
+                    make_p();
+                }
             }
 #pragma unroll
             for (int sb = 0; sb < NSUB; sb++)
 #pragma unroll
                 for (int kk = 0; kk < 2; kk++) op_cur[sb][kk] = op_next[sb][kk];
-            // all copies but those of the last LA - 1 steps have landed; the barrier publishes them
-            wait_vmcnt<OPS*(C::LA - 1)>();
+            // The barrier publishes the copies that the next step reads.  Copies complete in issue
+            // order (Q rows, then the bias slice of the same step).  S_AHEAD: the next step reads the
+            // Q rows issued one step ago, so only the bias slice issued behind them and this step's
+            // copies may still be in flight; else everything but the last LA - 1 steps has landed.
+            if constexpr (S_AHEAD) wait_vmcnt<(BV ? C::BCH : 0) + OPS*(C::LA - 2)>();
+            else wait_vmcnt<OPS*(C::LA - 1)>();
             lds_barrier();
-        }
+        };
+#pragma unroll 1
+        for (int t = mb_first - 1; t <= n_mblocks; t++) s_step(t);
         };
         if (BIAS != 0 && bias_vec) s_loop(std::true_type{});
         else s_loop(std::false_type{});
@@ -719,24 +830,44 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
                     lds_copy_end(saved_m0);
                 }
             };
+            const bool live = t >= mb_first && t < n_mblocks;
+            const int m0 = t * BMI;
+            const float* delta_lds = reinterpret_cast<const float*>(smem + C::OFF_DELTA) + ((t < 0 ? 0 : t) % C::NDOB) * BMI;
+            const float* p_in = p_lds + (t & 1) * (C::P_BYTES / 4);
+            T8 a_cols[NA], a_rows[NR];
+            f32x4 del_in[NSUB][4], p_vals[NSUB][4];
+            auto load_ds_inputs = [&]() {
+#pragma unroll
+                for (int sb = 0; sb < NSUB; sb++)
+#pragma unroll
+                    for (int q4 = 0; q4 < 4; q4++) {
+                        del_in[sb][q4] = *reinterpret_cast<const f32x4*>(delta_lds + sb * 32 + 8 * q4 + 4 * g);
+                        p_vals[sb][q4] = *reinterpret_cast<const f32x4*>(p_in + ((sb * 4 + q4) * 64 + lane) * 4);
+                    }
+            };
             if constexpr (BIAS == 0) issue_copies();
-            if (C::DEFER_DK && t - 1 >= mb_first)  // dK^T += Q(t-1)^T dS(t-1)
-                gemm_cols(reinterpret_cast<const T*>(smem + ((t - 1) % C::NQB) * C::Q_BYTES), op_cur);
-            if constexpr (BIAS != 0) issue_copies();  // in the shadow of the MFMAs just issued
-            if (t >= mb_first && t < n_mblocks) {
-                const int m0 = t * BMI;
+            // operands of both products up front: Q(t-1)^T for dK, the rows of dO(t) for dP
+            if constexpr (C::DEFER_DK) load_cols(q_tile(t - 1), a_cols);
+            load_rows(do_tile(t), a_rows);
+            if constexpr (PRELOAD && BIAS == 0) __builtin_amdgcn_sched_barrier(0);
+            if constexpr (BIAS != 0) issue_copies();  // behind the reads, whose round trip they cover
+            if (C::DEFER_DK && t - 1 >= mb_first) mma_cols(a_cols, op_cur);  // dK^T += Q(t-1)^T dS(t-1)
+            if (live) {
                 f32x16 sacc[NSUB];
-                gemm_rows(reinterpret_cast<const T*>(smem + C::OFF_DO + (t % C::NDOB) * C::Q_BYTES), sacc);
+                if constexpr (PRELOAD) {
+                    load_ds_inputs();  // land while the products run
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                mma_rows(a_rows, sacc);
+                if constexpr (!PRELOAD) load_ds_inputs();
                 // ---- dS = P (dP - delta) (flash_attention.py:303-308) ----
-                const float* delta_lds = reinterpret_cast<const float*>(smem + C::OFF_DELTA) + (t % C::NDOB) * BMI;
-                const float* p_in = p_lds + (t & 1) * (C::P_BYTES / 4);
 #pragma unroll
                 for (int sb = 0; sb < NSUB; sb++) {
 #pragma unroll
                     for (int q4 = 0; q4 < 4; q4++) {
                         const int ml0 = sb * 32 + 8 * q4 + 4 * g;
-                        const f32x4 del4 = *reinterpret_cast<const f32x4*>(delta_lds + ml0);
-                        const f32x4 p4 = *reinterpret_cast<const f32x4*>(p_in + ((sb * 4 + q4) * 64 + lane) * 4);
+                        const f32x4 del4 = del_in[sb][q4];
+                        const f32x4 p4 = p_vals[sb][q4];
                         T4 d4;
 #pragma unroll
                         for (int e = 0; e < 4; e++) {
@@ -779,8 +910,10 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
                         }
                     }
                 }
-                if (!C::DEFER_DK)  // dK^T += Q(t)^T dS(t)
-                    gemm_cols(reinterpret_cast<const T*>(smem + (t % C::NQB) * C::Q_BYTES), op_cur);
+                if constexpr (!C::DEFER_DK) {  // dK^T += Q(t)^T dS(t)
+                    load_cols(q_tile(t), a_cols);
+                    mma_cols(a_cols, op_cur);
+                }
             }
             if constexpr (COPIES > 0) wait_vmcnt<COPIES*(C::LA - 1)>();
             lds_barrier();
@@ -793,7 +926,6 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
             dp_loop(std::false_type{});
         }
     }
-
     // ---- dV (S-wave) or dK (dP-wave) of this wave's 32 keys (flash_attention.py:449-454) ----
     if (my_n < N) {
         T* dst = s_wave ? reinterpret_cast<T*>(p.dv) + (int64_t)b * p.sdv.b + (int64_t)h * p.sdv.h + (int64_t)my_n * p.sdv.s
@@ -852,14 +984,16 @@ template <typename T, int D> static hipError_t launch_all(const BwdParams& p, in
     if (stages & 4) {
         dim3 qgrid((unsigned)(p.n_mtiles * p.B * p.H));
         // dBias in fp32 or in the element type of q, written a moment ago by the key-tile kernel in
-        // rows of whole 16-byte chunks, is the dS the dQ product needs
+        // rows of whole 16-byte chunks, is the dS the dQ product needs.  Only when that kernel ran in
+        // this very call (or the caller vouches for the contents of dbias, bit 8) is it read.
         constexpr int DS_BIAS = __is_same(T, _Float16) ? 2 : 3;
-        if (dbias && bias == DS_BIAS && p.dbias_vec) {
+        const bool ds_valid = (stages & 2) || (stages & 8);
+        if (ds_valid && dbias && bias == DS_BIAS && p.dbias_vec) {
             if (causal) hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, DS_BIAS, true, true>), qgrid, dim3(256), 0, st, p);
             else hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, DS_BIAS, false, true>), qgrid, dim3(256), 0, st, p);
             return hipGetLastError();
         }
-        if (dbias && bias == 4 && p.dbias_vec) {
+        if (ds_valid && dbias && bias == 4 && p.dbias_vec) {
             if (causal) hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, 4, true, true>), qgrid, dim3(256), 0, st, p);
             else hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, 4, false, true>), qgrid, dim3(256), 0, st, p);
             return hipGetLastError();
@@ -883,22 +1017,16 @@ template <typename T, int D> static hipError_t launch_all(const BwdParams& p, in
     return e;
 }
 
-template <typename T> static hipError_t launch_d(const BwdParams& p, int D, int bias, bool causal, bool dbias, int stages, hipStream_t st) {
-    switch (D) {
-        case 16: return launch_all<T, 16>(p, bias, causal, dbias, stages, st);
-        case 32: return launch_all<T, 32>(p, bias, causal, dbias, stages, st);
-        case 64: return launch_all<T, 64>(p, bias, causal, dbias, stages, st);
-        case 128: return launch_all<T, 128>(p, bias, causal, dbias, stages, st);
-        case 256: return launch_all<T, 256>(p, bias, causal, dbias, stages, st);
-    }
-    return hipErrorNotSupported;
+// This file is compiled once per head dimension (-DFA_HEAD_DIM=16 ... 256); each object exports
+// launch_bwd_d<FA_HEAD_DIM>.
+#ifndef FA_HEAD_DIM
+#error "compile with -DFA_HEAD_DIM=<16|32|64|128|256>"
+#endif
+template <int D> hipError_t launch_bwd_d(const BwdParams& p, int dtype, int bias, bool causal, bool dbias, int stages, hipStream_t st);
+template <> hipError_t launch_bwd_d<FA_HEAD_DIM>(const BwdParams& p, int dtype, int bias, bool causal, bool dbias, int stages, hipStream_t st) {
+    if (dtype == 0) return launch_all<_Float16, FA_HEAD_DIM>(p, bias, causal, dbias, stages, st);
+    return launch_all<__bf16, FA_HEAD_DIM>(p, bias, causal, dbias, stages, st);
 }
-
-hipError_t launch_bwd(const BwdParams& p, int D, int dtype, int bias, bool causal, bool dbias, int stages, hipStream_t st) {
-    if (dtype == 0) return launch_d<_Float16>(p, D, bias, causal, dbias, stages, st);
-    return launch_d<__bf16>(p, D, bias, causal, dbias, stages, st);
-}
-
-int bwd_block_n(int) { return 128; }
 
 }  // namespace fa
+

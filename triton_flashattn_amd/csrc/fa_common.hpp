@@ -88,11 +88,28 @@ __device__ __forceinline__ int tr_offset(int lane, int row0, int col0, int strid
     int s = lane & 15;
     return (row0 + (s >> 2)) * stride + col0 + ((lane >> 4) & 1) * 16 + (s & 3) * 4;
 }
+// The same two reads by LDS byte address (a 32-bit integer) instead of by pointer
+__device__ __forceinline__ i32x4 lds_read16_at(unsigned addr) {
+    typedef const i32x4 __attribute__((address_space(3))) * lds_ptr;
+    return *(lds_ptr)(uintptr_t)addr;
+}
+__device__ __forceinline__ i16x4 lds_read_tr4_at(unsigned addr) {
+    typedef i16x4 __attribute__((address_space(3))) * lds_ptr;
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(uintptr_t)addr);
+}
 // Row-major LDS tile of 16-bit elements, D per row, no padding; the 16-byte chunks of a row are
 // XOR-swizzled by a function of the row so that both 16-byte row reads (lane = row) and 4-row
 // column gathers (ds_read_b64_tr_b16) are free of bank conflicts.
+//
+// Operand fetches by address.  A tile starts at a multiple of its row length in bytes, so the
+// XOR of the swizzle and the step along the head dim only touch address bits below the row
+// stride: the address of a lane's chunk is (tile + L) ^ step + rows, with ONE per-lane constant
+// L per access pattern (rows_lane for row operands, cols_lane for column gathers), a
+// compile-time `step`, and a compile-time row term that goes into the offset field of the read.
+// A kernel so keeps two address constants per lane instead of one per read.
 template <int D> struct Swz {
     static constexpr int CPR = D / 8;  // chunks per row
+    static constexpr int RB = 2 * D;   // bytes per row
     __device__ static __forceinline__ int f(int row) {
         if (CPR >= 16) return ((row & 3) << 2) | ((row >> 2) & 3);
         if (CPR == 8) return (((row >> 1) & 1) << 2) | ((row >> 2) & 3);
@@ -110,6 +127,32 @@ template <int D> struct Swz {
         const int col = (col0 + ((lane >> 4) & 1) * 16 + (s & 3) * 4) & (D - 1);
         i16x4 lo = lds_read_tr4(tile + off(row, col));
         i16x4 hi = lds_read_tr4(tile + off(row + 8, col));
+        typedef short i16x8 __attribute__((ext_vector_type(8)));
+        return __builtin_bit_cast(V8, (i16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    }
+    // Row operand: lane l reads row (rows + l%32), head-dim elements 16 ks + 8 (l/32) .. + 7.
+    // rows_lane(lane) is L; `rows` is a multiple of 32 known at compile time.
+    __device__ static __forceinline__ unsigned rows_lane(int lane) {
+        const int r = lane & 31, g = lane >> 5;
+        return (unsigned)(r * RB + 16 * (g ^ f(r)));
+    }
+    template <typename V8> __device__ static __forceinline__ V8 row8_at(unsigned tile_plus_l, int rows, int ks) {
+        return __builtin_bit_cast(V8, lds_read16_at((tile_plus_l ^ (unsigned)(32 * ks)) + (unsigned)(rows * RB)));
+    }
+    // Column operand (what col8 returns) for head-dim block db (32 wide) and rows row0 .. row0 + 15,
+    // row0 a multiple of 16 known at compile time.  The second gather sits 8 rows further down,
+    // where the swizzle differs by one fixed bit.
+    __device__ static __forceinline__ unsigned cols_lane(int lane) {
+        const int g = lane >> 5, s = lane & 15;
+        const int rl = 4 * g + (s >> 2);
+        const int col = (((lane >> 4) & 1) * 16 + (s & 3) * 4) & (D - 1);
+        return (unsigned)(rl * RB + 16 * ((col >> 3) ^ f(rl)) + 2 * (col & 7));
+    }
+    template <typename V8> __device__ static __forceinline__ V8 col8_at(unsigned tile_plus_l, int row0, int db) {
+        constexpr unsigned H = CPR == 2 ? 16u : 32u;  // f(row + 8) ^ f(row), as a byte offset
+        const unsigned x = (unsigned)((64 * db) & (RB - 1));
+        i16x4 lo = lds_read_tr4_at((tile_plus_l ^ x) + (unsigned)(row0 * RB));
+        i16x4 hi = lds_read_tr4_at((tile_plus_l ^ x ^ H) + (unsigned)((row0 + 8) * RB));
         typedef short i16x8 __attribute__((ext_vector_type(8)));
         return __builtin_bit_cast(V8, (i16x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
     }
@@ -146,10 +189,15 @@ __device__ __forceinline__ unsigned lds_addr_of(const void* p) {
 }
 // A wave-uniform pointer, forced into scalar registers (the compiler may have computed it with
 // vector instructions, and an inline-asm scalar operand is not moved there by itself).
+// A vector-memory instruction that reads an SGPR written by a VALU instruction (v_readfirstlane
+// here) needs five wait states in between.  The compiler inserts them for its own instructions
+// but cannot see into inline assembly, so they are added here, tied to the two registers so that
+// they sit between the write and every use.
 __device__ __forceinline__ uint64_t uniform_ptr(const void* p) {
     const uint64_t b = (uint64_t)(uintptr_t)p;
-    const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)b);
-    const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(b >> 32));
+    unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)b);
+    unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(b >> 32));
+    asm volatile("s_nop 4" : "+s"(lo), "+s"(hi));
     return ((uint64_t)hi << 32) | lo;
 }
 // between lds_copy_begin() and lds_copy_end(): 16 bytes per lane from base + voff to lds_addr + 16 l

@@ -302,23 +302,15 @@ template <typename T, int D> static hipError_t launch_bias(const FwdParams& p, i
     return hipErrorInvalidValue;
 }
 
-template <typename T> static hipError_t launch_d(const FwdParams& p, int D, int bias, bool causal, hipStream_t st) {
-    switch (D) {
-        case 16: return launch_bias<T, 16>(p, bias, causal, st);
-        case 32: return launch_bias<T, 32>(p, bias, causal, st);
-        case 64: return launch_bias<T, 64>(p, bias, causal, st);
-        case 128: return launch_bias<T, 128>(p, bias, causal, st);
-        case 256: return launch_bias<T, 256>(p, bias, causal, st);
-    }
-    return hipErrorInvalidValue;
+// This file is compiled once per head dimension (-DFA_HEAD_DIM=16 ... 256); each object exports
+// launch_fwd_d<FA_HEAD_DIM>.  dtype: 0 = fp16, 1 = bf16.  The caller has validated every argument.
+#ifndef FA_HEAD_DIM
+#error "compile with -DFA_HEAD_DIM=<16|32|64|128|256>"
+#endif
+template <int D> hipError_t launch_fwd_d(const FwdParams& p, int dtype, int bias, bool causal, hipStream_t st);
+template <> hipError_t launch_fwd_d<FA_HEAD_DIM>(const FwdParams& p, int dtype, int bias, bool causal, hipStream_t st) {
+    if (dtype == 0) return launch_bias<_Float16, FA_HEAD_DIM>(p, bias, causal, st);
+    return launch_bias<__bf16, FA_HEAD_DIM>(p, bias, causal, st);
 }
-
-// dtype: 0 = fp16, 1 = bf16.  The caller has validated every argument.
-hipError_t launch_fwd(const FwdParams& p, int D, int dtype, int bias, bool causal, hipStream_t st) {
-    if (dtype == 0) return launch_d<_Float16>(p, D, bias, causal, st);
-    return launch_d<__bf16>(p, D, bias, causal, st);
-}
-
-int fwd_block_m() { return 128; }
 
 }  // namespace fa

@@ -104,11 +104,11 @@ class _HipBackend:
         a.p = self._problem(q, k, bias, causal, sm_scale)
         if workspace is None:
             workspace = self.bwd_workspace(q, k, bias, causal, sm_scale)
-        nbytes = workspace.numel()
         a.q, a.k, a.v, a.o, a.dout, a.lse = (q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
                                              do.data_ptr(), lse.data_ptr())
         a.dq, a.dk, a.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
-        a.workspace, a.workspace_bytes = workspace.data_ptr(), nbytes
+        if workspace is not None:
+            a.workspace, a.workspace_bytes = workspace.data_ptr(), workspace.numel()
         a.q_strides, a.k_strides, a.v_strides, a.o_strides = _strides4(q), _strides4(k), _strides4(v), _strides4(o)
         a.do_strides, a.dq_strides, a.dk_strides, a.dv_strides = (_strides4(do), _strides4(dq), _strides4(dk),
                                                                   _strides4(dv))

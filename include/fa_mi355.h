@@ -47,7 +47,8 @@ enum fa_status {
     FA_ERR_LAYOUT = -5,      /* alignment or stride rule above violated */
     FA_ERR_WORKSPACE = -6,   /* workspace NULL or smaller than fa_bwd_workspace_bytes() */
     FA_ERR_UNSUPPORTED = -7, /* combination not built into this library */
-    FA_ERR_LAUNCH = -8       /* the HIP runtime rejected a launch (hipGetLastError) */
+    FA_ERR_LAUNCH = -8,      /* the HIP runtime rejected a launch (hipGetLastError) */
+    FA_ERR_TOO_LARGE = -9    /* fa_bwd_noalloc: B * H * M exceeds FA_NOALLOC_MAX_ROWS */
 };
 
 /* Problem description shared by forward and backward.  Strides are in elements. */
@@ -123,6 +124,17 @@ enum fa_bwd_stage {
  * FA_STAGE_DQ alone recomputes dS from q, k, v and the bias and never reads dbias, unless
  * FA_STAGE_DQ_FROM_DBIAS is added.  Both routes agree within the rounding of dS to 16 bits. */
 int fa_bwd_stages(const fa_bwd_args *args, void *stream, int stages);
+
+/* fa_bwd for callers that cannot allocate device memory (HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  No counterpart in the reference, whose launcher allocates
+ * delta itself (flash_attention.py:689).  args->workspace and args->workspace_bytes are ignored:
+ * delta lives in a static device array of FA_NOALLOC_MAX_ROWS floats (4 MiB per GPU, held until
+ * the process ends), so B * H * M must not exceed FA_NOALLOC_MAX_ROWS (FA_ERR_TOO_LARGE
+ * otherwise).  The call allocates and frees nothing.  All calls on one GPU share the array:
+ * calls that may overlap on one GPU (different streams, different threads) race on it; on one
+ * stream they are ordered and safe.  Results are bit-identical to fa_bwd. */
+#define FA_NOALLOC_MAX_ROWS (1 << 20)
+int fa_bwd_noalloc(const fa_bwd_args *args, void *stream);
 
 #ifdef __cplusplus
 }

@@ -221,3 +221,8 @@ def test_abi_status_codes_and_workspace():
     b.dbias = None
     assert lib.fa_bwd_stages(ctypes.byref(b), None, 16) == -7                       # unknown stage bit
     assert lib.fa_bwd_stages(ctypes.byref(b), None, _native.FA_STAGE_DQ_FROM_DBIAS) == -7   # modifier alone
+    big = _native.FaBwdArgs()
+    big.p = _native.FaProblem(B=1, H=1, M=_native.FA_NOALLOC_MAX_ROWS + 1, N=8, D=64, dtype=_native.FA_BF16,
+                              bias_dtype=0, causal=0, sm_scale=0.1)
+    assert lib.fa_bwd_noalloc(ctypes.byref(big), None) == _native.FA_ERR_TOO_LARGE  # beyond the static scratch
+    assert lib.fa_bwd_noalloc(None, None) == -1

@@ -46,8 +46,11 @@ class FaBwdArgs(ctypes.Structure):
     ]
 
 
-EXPORTS = ("fa_abi_version", "fa_strerror", "fa_fwd", "fa_bwd_workspace_bytes", "fa_bwd", "fa_bwd_stages")
+EXPORTS = ("fa_abi_version", "fa_strerror", "fa_fwd", "fa_bwd_workspace_bytes", "fa_bwd", "fa_bwd_stages",
+           "fa_bwd_noalloc")
 FA_STAGE_PREP, FA_STAGE_MAIN, FA_STAGE_DQ, FA_STAGE_ALL, FA_STAGE_DQ_FROM_DBIAS = 1, 2, 4, 7, 8
+FA_NOALLOC_MAX_ROWS = 1 << 20
+FA_ERR_TOO_LARGE = -9
 
 _lib = None
 
@@ -78,6 +81,8 @@ def load():
     lib.fa_bwd.argtypes = [ctypes.POINTER(FaBwdArgs), ctypes.c_void_p]
     lib.fa_bwd_stages.restype = ctypes.c_int
     lib.fa_bwd_stages.argtypes = [ctypes.POINTER(FaBwdArgs), ctypes.c_void_p, ctypes.c_int]
+    lib.fa_bwd_noalloc.restype = ctypes.c_int
+    lib.fa_bwd_noalloc.argtypes = [ctypes.POINTER(FaBwdArgs), ctypes.c_void_p]
     if lib.fa_abi_version() != ABI_VERSION:
         raise NativeLibraryError("libfa_mi355.so has ABI %d, expected %d" % (lib.fa_abi_version(), ABI_VERSION))
     _lib = lib

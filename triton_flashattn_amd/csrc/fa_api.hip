@@ -2,6 +2,8 @@
 // Host code only; the kernels live in fa_fwd.hip and fa_bwd.hip.
 #include <hip/hip_runtime.h>
 
+#include <mutex>
+
 #include "../../include/fa_mi355.h"
 #include "fa_params.hpp"
 
@@ -42,6 +44,34 @@ static hipError_t launch_bwd(const BwdParams& p, int D, int dtype, int bias, boo
 // query rows per work-group of the forward and dQ kernels; keys per work-group of the dK/dV kernel
 static int fwd_block_m() { return 128; }
 static int bwd_block_n(int) { return 128; }
+}  // namespace fa
+
+// Scratch of fa_bwd_noalloc: delta, one float per (batch, head, query row).  Every GPU the library
+// runs on holds its own copy of this array until the process ends.  In host code the name is only
+// a handle; the device address comes from hipGetSymbolAddress (scratch_on_current_device).
+static __device__ __align__(256) float scratch[FA_NOALLOC_MAX_ROWS];
+
+namespace fa {
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static float* g_scratch_ptr[kMaxDevices];  // device address of `scratch`, per device
+
+// Address of this device's copy of `scratch`, looked up once per device with that device current.
+// This function has external linkage on purpose: the compiler gives a static device variable a
+// symbol the runtime can find only when a host function with external linkage refers to it.
+float* scratch_on_current_device() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess) return nullptr;
+        g_scratch_ptr[dev] = static_cast<float*>(ptr);
+    }
+    return g_scratch_ptr[dev];
+}
+
 }  // namespace fa
 
 namespace {
@@ -121,6 +151,7 @@ const char* fa_strerror(int status) {
         case FA_ERR_WORKSPACE: return "workspace is NULL, misaligned or smaller than fa_bwd_workspace_bytes()";
         case FA_ERR_UNSUPPORTED: return "combination not built into this library";
         case FA_ERR_LAUNCH: return "HIP kernel launch failed";
+        case FA_ERR_TOO_LARGE: return "fa_bwd_noalloc: B * H * M exceeds FA_NOALLOC_MAX_ROWS";
     }
     return "unknown status";
 }
@@ -217,5 +248,15 @@ extern "C" {
 int fa_bwd_stages(const fa_bwd_args* a, void* stream, int stages) { return bwd_enqueue(a, stream, stages, nullptr); }
 
 int fa_bwd(const fa_bwd_args* a, void* stream) { return bwd_enqueue(a, stream, FA_STAGE_ALL, nullptr); }
+
+int fa_bwd_noalloc(const fa_bwd_args* a, void* stream) {
+    if (!a) return FA_ERR_NULL;
+    int st = check_problem(a->p);
+    if (st != FA_OK) return st;
+    if ((int64_t)a->p.B * a->p.H * a->p.M > (int64_t)FA_NOALLOC_MAX_ROWS) return FA_ERR_TOO_LARGE;
+    float* delta = fa::scratch_on_current_device();
+    if (!delta) return FA_ERR_LAUNCH;
+    return bwd_enqueue(a, stream, FA_STAGE_ALL, delta);
+}
 
 }  // extern "C"

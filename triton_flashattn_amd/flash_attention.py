@@ -97,12 +97,17 @@ class _HipBackend:
         return torch.empty(nbytes, dtype=torch.uint8, device=q.device)
 
     def bwd(self, do, q, k, v, o, bias, causal, sm_scale, lse, dq, dk, dv, dbias,
-            stages=_native.FA_STAGE_ALL, workspace=None):
+            stages=_native.FA_STAGE_ALL, workspace=None, noalloc=False):
+        """noalloc: call fa_bwd_noalloc (delta in the library's static device array, nothing is
+        allocated; all stages)."""
         dev = self._require_gpu(do, q, k, v, o, bias, lse, dq, dk, dv, dbias)
         lib = _native.load()
         a = _native.FaBwdArgs()
         a.p = self._problem(q, k, bias, causal, sm_scale)
-        if workspace is None:
+        if noalloc:
+            if workspace is not None or stages != _native.FA_STAGE_ALL:
+                raise ValueError("fa_bwd_noalloc takes no workspace and runs every stage")
+        elif workspace is None:
             workspace = self.bwd_workspace(q, k, bias, causal, sm_scale)
         a.q, a.k, a.v, a.o, a.dout, a.lse = (q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(),
                                              do.data_ptr(), lse.data_ptr())
@@ -120,7 +125,10 @@ class _HipBackend:
             a.dbias_strides = _strides4(dbias)
         with torch.cuda.device(dev):
             stream = torch.cuda.current_stream(dev).cuda_stream
-            _native.check(lib.fa_bwd_stages(ctypes.byref(a), ctypes.c_void_p(stream), int(stages)))
+            if noalloc:
+                _native.check(lib.fa_bwd_noalloc(ctypes.byref(a), ctypes.c_void_p(stream)))
+            else:
+                _native.check(lib.fa_bwd_stages(ctypes.byref(a), ctypes.c_void_p(stream), int(stages)))
             # the workspace is only touched by work already enqueued on this stream; the caching
             # allocator re-issues it to later work on the same stream only, so it may be dropped
 

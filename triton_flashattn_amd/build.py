@@ -4,6 +4,7 @@ Usage: python -m triton_flashattn_amd.build [-j N]
 hipcc cross-compiles without a GPU, so this runs anywhere the ROCm toolchain is installed.
 """
 import os
+import re
 import subprocess
 import sys
 from concurrent.futures import ThreadPoolExecutor
@@ -20,6 +21,8 @@ FLAGS = [
     # packed fp32 VALU ops are kept out of the generated code on purpose
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
+    # one remark block per kernel with its register, scratch and LDS use; read by _scratch_users
+    "-Rpass-analysis=kernel-resource-usage",
 ]
 
 
@@ -32,17 +35,40 @@ def _compile(unit):
     log = "\n".join(l for l in (res.stdout + res.stderr).splitlines() if "packed-fp32-ops" not in l)
     if res.returncode != 0:
         raise RuntimeError("hipcc failed for %s (D=%s):\n%s" % (src, d, log))
-    return obj, log
+    return obj, log, d
+
+
+def _scratch_users(log):
+    """(kernel, VGPRs, scratch bytes per lane) of every kernel in a compile log that spills."""
+    out, name, vgprs = [], None, None
+    for line in log.splitlines():
+        m = re.search(r"Function Name: (\S+)", line)
+        if m:
+            name, vgprs = m.group(1), None
+        m = re.search(r" VGPRs: (\d+)", line)
+        if m:
+            vgprs = int(m.group(1))
+        m = re.search(r"ScratchSize \[bytes/lane\]: (\d+)", line)
+        if m and name and int(m.group(1)) > 0:
+            out.append((name, vgprs, int(m.group(1))))
+    return out
 
 
 def build(jobs=8, verbose=False):
     with ThreadPoolExecutor(max_workers=max(1, jobs)) as ex:
         results = list(ex.map(_compile, UNITS))
-    objs = [o for o, _ in results]
+    objs = [o for o, _, _ in results]
+    # A kernel that spills registers to scratch runs its spill traffic through the same queue as
+    # the hand-counted direct-to-LDS copies: up to head dim 128 no kernel may do that.  The D = 256
+    # kernels are known to spill (correct, slow) and are only reported.
+    spills = [(d, k, v, b) for _, log, d in results for k, v, b in _scratch_users(log)]
+    bad = [x for x in spills if x[0] is not None and x[0] <= 128]
     if verbose:
-        for _, log in results:
-            if log.strip():
-                print(log)
+        for d, k, v, b in spills:
+            print("scratch: D=%s %s: %d VGPRs, %d bytes/lane" % (d, k, v, b))
+    if bad:
+        raise RuntimeError("kernels with head dim <= 128 spill registers:\n" + "\n".join(
+            "  D=%s %s: %s VGPRs, %d bytes/lane of scratch" % x for x in bad))
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:

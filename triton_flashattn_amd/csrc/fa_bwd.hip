@@ -65,7 +65,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_
     typedef typename BiasElem<BIAS>::type E;
     constexpr int BM = C::BM, BK = C::BK, OS = C::OS, CPR = C::CPR;
 
-    __shared__ __align__(16) unsigned char smem[C::LDS_BYTES];
+    __shared__ __align__(1024) unsigned char smem[C::LDS_BYTES];
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
@@ -120,6 +120,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_
 #pragma unroll
         for (int i = 0; i < 16; i++) dq_acc[db][i] = 0.f;
 
+    const unsigned rows_l = SW::rows_lane(lane), cols_l = SW::cols_lane(lane);
     KeyStream<T, D, BIAS, !FROM_DS> ks_;
     ks_.init(smem, kp, vp, bp, p.sk.s, p.sv.s, FROM_DS ? p.sdbias.m : p.sbias.m, FROM_DS ? p.sdbias.n : p.sbias.n, M, N,
              mw, wave, lane);
@@ -132,8 +133,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_
         constexpr bool BV = decltype(bv_tag)::value;
         const int n0 = k * BK;
         ks_.template begin_step<BV>(k);
-        const T* k_lds = ks_.k_lds(k);
-        const T* v_lds = ks_.v_lds(k);
+        const unsigned k_tile = ks_.k_addr(k), v_tile = ks_.v_addr(k);  // operand reads by address
         const unsigned char* b_lds = ks_.b_lds(k);
         static_assert(BIAS == 0 || C::NH == 1, "a bias slot covers one 32-key block");
         // The step is consumed 32 keys at a time, so that only one 32 x 32 score block is live.
@@ -178,7 +178,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_
             for (int i = 0; i < 16; i++) s[i] = 0.f;
 #pragma unroll
             for (int ks = 0; ks < C::KSTEPS; ks++) {
-                T8 a = as_vec<T8>(lds_read16(k_lds + SW::off(nh + r, ks * 16 + 8 * g)));
+                T8 a = SW::template row8_at<T8>(k_tile + rows_l, nh, ks);
                 s = mfma32(a, qreg[ks], s);
             }
 
@@ -188,7 +188,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_
             for (int i = 0; i < 16; i++) dp[i] = 0.f;
 #pragma unroll
             for (int ks = 0; ks < C::KSTEPS; ks++) {
-                T8 a = as_vec<T8>(lds_read16(v_lds + SW::off(nh + r, ks * 16 + 8 * g)));
+                T8 a = SW::template row8_at<T8>(v_tile + rows_l, nh, ks);
                 dp = mfma32(a, doreg[ks], dp);
             }
             if (nb == 0) ks_.template issue_ahead<BV>(k);  // in the shadow of the MFMAs just issued
@@ -256,7 +256,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_
             for (int kk = 0; kk < 2; kk++) {
 #pragma unroll
                 for (int db = 0; db < C::DB; db++) {
-                    T8 a = SW::template col8<T8>(k_lds, lane, nh + kk * 16, db * 32);
+                    T8 a = SW::template col8_at<T8>(k_tile + cols_l, nh + kk * 16, db);
                     dq_acc[db] = mfma32(a, dsb[kk], dq_acc[db]);
                 }
             }

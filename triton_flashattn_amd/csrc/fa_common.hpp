@@ -332,6 +332,9 @@ template <typename T, int D, int BIAS, bool WITH_V = true> struct KeyStream {
     __device__ __forceinline__ const T* k_lds(int k) const { return reinterpret_cast<const T*>(smem + (k % C::NKV) * C::STEP_BYTES); }
     __device__ __forceinline__ const T* v_lds(int k) const { return reinterpret_cast<const T*>(smem + (C::NKV + k % C::NKV) * C::STEP_BYTES); }
     __device__ __forceinline__ unsigned char* b_lds(int k) const { return bias_lds + (k % C::NBS) * C::BSLOT; }
+    // the K and V slots by LDS byte address (scalar), for the operand reads by address of Swz
+    __device__ __forceinline__ unsigned k_addr(int k) const { return lds_kv + (unsigned)((k % C::NKV) * C::STEP_BYTES); }
+    __device__ __forceinline__ unsigned v_addr(int k) const { return lds_kv + (unsigned)((C::NKV + k % C::NKV) * C::STEP_BYTES); }
     // byte offset of bias (row, key .. key + 3) inside a slot
     __device__ static __forceinline__ int b_off(int row, int key) {
         const int byte = key * C::ES;

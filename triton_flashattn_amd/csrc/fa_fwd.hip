@@ -35,7 +35,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_
     typedef typename BiasElem<BIAS>::type E;
     constexpr int BM = C::BM, BK = C::BK, OS = C::OS, CPR = C::CPR;
 
-    __shared__ __align__(16) unsigned char smem[C::LDS_BYTES];
+    __shared__ __align__(1024) unsigned char smem[C::LDS_BYTES];
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
@@ -79,6 +79,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_
 #pragma unroll
         for (int i = 0; i < 16; i++) o_acc[db][i] = 0.f;
 
+    const unsigned rows_l = SW::rows_lane(lane), cols_l = SW::cols_lane(lane);
     KeyStream<T, D, BIAS> ks_;
     ks_.init(smem, kp, vp, bp, p.sk.s, p.sv.s, p.sbias.m, p.sbias.n, M, N, mw, wave, lane);
 
@@ -90,8 +91,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_
         constexpr bool BV = decltype(bv_tag)::value;
         const int n0 = k * BK;
         ks_.template begin_step<BV>(k);
-        const T* k_lds = ks_.k_lds(k);
-        const T* v_lds = ks_.v_lds(k);
+        const unsigned k_rows = ks_.k_addr(k) + rows_l, v_cols = ks_.v_addr(k) + cols_l;  // operand reads by address
         const unsigned char* b_lds = ks_.b_lds(k);
         static_assert(BIAS == 0 || C::NH == 1, "a bias slot covers one 32-key block");
         // The step is consumed 32 keys at a time, each block with its own softmax step.  In interior
@@ -106,7 +106,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_
                 for (int i = 0; i < 16; i++) s_pre[nb][i] = 0.f;
 #pragma unroll
                 for (int ks = 0; ks < C::KSTEPS; ks++) {
-                    T8 a = as_vec<T8>(lds_read16(k_lds + SW::off(nb * 32 + r, ks * 16 + 8 * g)));
+                    T8 a = SW::template row8_at<T8>(k_rows, nb * 32, ks);
                     s_pre[nb] = mfma32(a, qreg[ks], s_pre[nb]);
                 }
             }
@@ -132,7 +132,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_
             for (int i = 0; i < 16; i++) s[i] = 0.f;
 #pragma unroll
             for (int ks = 0; ks < C::KSTEPS; ks++) {
-                T8 a = as_vec<T8>(lds_read16(k_lds + SW::off(nh + r, ks * 16 + 8 * g)));
+                T8 a = SW::template row8_at<T8>(k_rows, nh, ks);
                 s = mfma32(a, qreg[ks], s);
             }
             if (nb == 0) ks_.template issue_ahead<BV>(k);  // in the shadow of the MFMAs just issued
@@ -225,7 +225,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_
                 }
 #pragma unroll
                 for (int db = 0; db < C::DB; db++) {
-                    T8 a = SW::template col8<T8>(v_lds, lane, nh + kk * 16, db * 32);
+                    T8 a = SW::template col8_at<T8>(v_cols, nh + kk * 16, db);
                     o_acc[db] = mfma32(a, pb[kk], o_acc[db]);
                 }
             }

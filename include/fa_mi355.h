@@ -29,14 +29,21 @@
 extern "C" {
 #endif
 
-#define FA_ABI_VERSION 1
+#define FA_ABI_VERSION 2
 
 /* element type of q, k, v, o and their gradients */
 enum fa_dtype { FA_F16 = 0, FA_BF16 = 1 };
 
 /* element type of bias (and of dbias, which always has the type of bias);
- * FA_BIAS_BOOL is one byte per element, non-zero = keep (flash_attention.py:48-50) */
-enum fa_bias_dtype { FA_BIAS_NONE = 0, FA_BIAS_BOOL = 1, FA_BIAS_F16 = 2, FA_BIAS_BF16 = 3, FA_BIAS_F32 = 4 };
+ * FA_BIAS_BOOL is one byte per element, non-zero = keep (flash_attention.py:48-50).
+ * FA_BIAS_ALIBI has no counterpart in the reference, which needs such a bias materialized
+ * (README.md:9): `bias` points to H fp32 slopes and the kernels compute
+ *   bias[b, h, i, j] = -slope[h] * |i * N / M - j|
+ * from the indices; bias_strides are ignored, and dbias (when non-NULL) receives the H fp32 slope
+ * gradients, dslope[h] = sum over b, i, j of dS[b, h, i, j] * -|i * N / M - j|. */
+enum fa_bias_dtype {
+    FA_BIAS_NONE = 0, FA_BIAS_BOOL = 1, FA_BIAS_F16 = 2, FA_BIAS_BF16 = 3, FA_BIAS_F32 = 4, FA_BIAS_ALIBI = 5
+};
 
 enum fa_status {
     FA_OK = 0,
@@ -48,7 +55,7 @@ enum fa_status {
     FA_ERR_WORKSPACE = -6,   /* workspace NULL or smaller than fa_bwd_workspace_bytes() */
     FA_ERR_UNSUPPORTED = -7, /* combination not built into this library */
     FA_ERR_LAUNCH = -8,      /* the HIP runtime rejected a launch (hipGetLastError) */
-    FA_ERR_TOO_LARGE = -9    /* fa_bwd_noalloc: B * H * M exceeds FA_NOALLOC_MAX_ROWS */
+    FA_ERR_TOO_LARGE = -9    /* fa_bwd_noalloc: the problem exceeds FA_NOALLOC_MAX_ROWS */
 };
 
 /* Problem description shared by forward and backward.  Strides are in elements. */
@@ -72,7 +79,16 @@ typedef struct fa_fwd_args {
 
 /* _flash_attn_bwd: flash_attention.py:688-763.  dq, dk, dv (and dbias when non-NULL, i.e. when
  * the bias is trainable, flash_attention.py:693,799) are outputs and are fully overwritten:
- * unlike the reference's dbias they need no zero fill by the caller. */
+ * unlike the reference's dbias they need no zero fill by the caller.
+ *
+ * dbias of a float bias comes in two layouts, told apart by dbias_strides:
+ *   dense    (B, H, M, N), every stride of a dimension larger than 1 non-zero: dbias = dS, as the
+ *            reference stores it (flash_attention.py:307-308);
+ *   reduced  the gradient of a bias that was broadcast over the query rows, (B or 1, H or 1, 1, N):
+ *            dbias_strides[2] == 0, and dbias_strides[0] / [1] == 0 where the bias was broadcast over
+ *            batches / heads too.  The kernels sum dS over the rows (and a second small kernel over
+ *            the broadcast batches / heads), so no (B, H, M, N) gradient is ever written.  No
+ *            counterpart in the reference, which leaves that reduction to autograd. */
 typedef struct fa_bwd_args {
     fa_problem p;
     const void *q, *k, *v, *o, *dout, *bias;
@@ -96,7 +112,7 @@ const char *fa_strerror(int status);
 int fa_fwd(const fa_fwd_args *args, void *stream);
 
 /* Bytes of scratch the backward needs for this problem: delta, (B, H, M) fp32
- * (flash_attention.py:689).  Depends on B, H, M only. */
+ * (flash_attention.py:689), followed by the partial sums of the reduced dbias layouts. */
 size_t fa_bwd_workspace_bytes(const fa_problem *p);
 
 /* Enqueue the backward (delta, dK/dV/dBias/dQ) on `stream`.
@@ -128,8 +144,9 @@ int fa_bwd_stages(const fa_bwd_args *args, void *stream, int stages);
 /* fa_bwd for callers that cannot allocate device memory (HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc).  No counterpart in the reference, whose launcher allocates
  * delta itself (flash_attention.py:689).  args->workspace and args->workspace_bytes are ignored:
- * delta lives in a static device array of FA_NOALLOC_MAX_ROWS floats (4 MiB per GPU, held until
- * the process ends), so B * H * M must not exceed FA_NOALLOC_MAX_ROWS (FA_ERR_TOO_LARGE
+ * the scratch (delta and the partial sums of a reduced dbias) lives in a static device array
+ * of 2 * FA_NOALLOC_MAX_ROWS floats (8 MiB per GPU, held until the process ends), so neither
+ * B * H * M nor B * H * max(N, 4) may exceed FA_NOALLOC_MAX_ROWS (FA_ERR_TOO_LARGE
  * otherwise).  The call allocates and frees nothing.  All calls on one GPU share the array:
  * calls that may overlap on one GPU (different streams, different threads) race on it; on one
  * stream they are ordered and safe.  Results are bit-identical to fa_bwd. */

@@ -1,0 +1,203 @@
+"""GPU parity tests of what goes beyond the reference's contract: ALiBi computed in the kernels
+(no bias tensor), gradients of row-broadcast biases reduced in the kernels (no dense dBias), biases
+of lower rank, V with its own head dim, gradients nobody asked for, the torch.library operator.
+Each is checked against the fp32 oracle run on the materialised equivalent.  Tolerances as in
+test_gpu_parity.py."""
+import pytest
+import torch
+
+import triton_flashattn_amd.flash_attention as fa_mod
+from triton_flashattn_amd import (AlibiBias, flash_attention_fn, flash_attention_op,
+                                  flash_attention_qkvpacked_fn)
+from triton_flashattn_amd.flash_attention import _flash_attn_fwd
+from test_gpu_parity import GRAD_RTOL, OUT_ATOL, check, make_inputs, rel_l2, run_oracle, run_ours
+
+pytestmark = pytest.mark.gpu
+
+
+def _slopes(H, dev):
+    return (2.0 ** (-8.0 * (torch.arange(H, dtype=torch.float32) + 1) / H)).to(dev)
+
+
+# ---------------------------------------------------------------- ALiBi in the kernels
+@pytest.mark.parametrize("D", [16, 64, 128, 256])
+@pytest.mark.parametrize("causal", [False, True])
+def test_alibi_matches_oracle_on_the_materialised_bias(gpu_device, D, causal):
+    """bias[b, h, i, j] = -slope[h] |i N / M - j| formed from indices inside the kernels: out, dq, dk,
+    dv and the slope gradient against the oracle fed the same bias as an fp32 tensor."""
+    shapes = [(2, 200, 200, 4), (1, 129, 129, 3), (1, 384, 384, 2)] if causal else \
+             [(2, 200, 333, 4), (1, 96, 384, 3), (1, 300, 100, 2), (1, 1, 1, 1)]
+    for i, (B, M, N, H) in enumerate(shapes):
+        dtype = torch.bfloat16 if i % 2 == 0 else torch.float16
+        q, k, v, do, _ = make_inputs(gpu_device, B, M, N, H, D, dtype, None, seed=3 * D + i)
+        slopes = _slopes(H, gpu_device).requires_grad_(True)
+        dense = AlibiBias(slopes.detach()).materialize(M, N)
+        assert dense.shape == (1, H, M, N) and dense.dtype == torch.float32
+        ours = run_ours(q, k, v, do, AlibiBias(slopes), causal)
+        ref = run_oracle(q, k, v, do, dense.expand(B, H, M, N), causal)
+        check(ours, ref, "alibi D%d %s" % (D, (B, M, N, H)))
+        dist = dense / slopes.detach().view(1, H, 1, 1)          # -|i N / M - j|
+        want = (ref["dbias"] * dist).sum(dim=(0, 2, 3))
+        assert slopes.grad.shape == (H,)
+        assert rel_l2(slopes.grad, want) <= GRAD_RTOL, (D, B, M, N, H, slopes.grad, want)
+
+
+def test_alibi_is_deterministic_and_needs_no_gradient(gpu_device):
+    q, k, v, do, _ = make_inputs(gpu_device, 2, 500, 500, 4, 64, torch.bfloat16, None, seed=77)
+    slopes = _slopes(4, gpu_device)
+    runs = []
+    for _ in range(2):
+        s = slopes.clone().requires_grad_(True)
+        r = run_ours(q, k, v, do, AlibiBias(s), True)
+        runs.append((r["dq"], r["dk"], r["dv"], s.grad))
+    for a, b in zip(*runs):
+        assert torch.equal(a, b)
+    r = run_ours(q, k, v, do, AlibiBias(slopes), True)        # slopes that are not trained
+    assert torch.equal(r["dq"], runs[0][0]) and slopes.grad is None
+
+
+def test_alibi_packed_entry(gpu_device):
+    B, S, H, D = 2, 300, 4, 64
+    g = torch.Generator().manual_seed(8)
+    qkv = torch.randn(B, S, 3, H, D, generator=g).bfloat16().to(gpu_device).requires_grad_(True)
+    do = torch.randn(B, S, H, D, generator=g).bfloat16().to(gpu_device)
+    slopes = _slopes(H, gpu_device)
+    out = flash_attention_qkvpacked_fn(qkv, AlibiBias(slopes), True)
+    out.backward(do)
+    q, k, v = qkv.detach().unbind(2)
+    ref = run_oracle(q, k, v, do, AlibiBias(slopes).materialize(S, S).expand(B, H, S, S), True)
+    assert (out.float() - ref["out"]).abs().max().item() <= OUT_ATOL
+    for i, n in enumerate(("dq", "dk", "dv")):
+        assert rel_l2(qkv.grad[:, :, i], ref[n]) <= GRAD_RTOL, n
+
+
+# ---------------------------------------------------------------- broadcast biases
+@pytest.mark.parametrize("D", [32, 128])
+@pytest.mark.parametrize("bdt", [torch.bfloat16, torch.float16, torch.float32])
+def test_row_broadcast_bias_gradient_is_reduced_in_the_kernels(gpu_device, D, bdt):
+    """A bias that is the same for every query row ((1, H, 1, N), (B, 1, 1, N), (N,) ...): its
+    gradient is the column sum of dS, accumulated in the kernels; no (B, H, M, N) tensor exists."""
+    B, M, N, H = 2, 300, 333, 3
+    for i, shape in enumerate([(1, H, 1, N), (B, 1, 1, N), (B, H, 1, N), (1, 1, 1, N), (N,), (H, 1, N)]):
+        for causal in (False, True):
+            Mc = N if causal else M
+            q, k, v, do, _ = make_inputs(gpu_device, B, Mc, N, H, D, torch.bfloat16, None, seed=5 * D + i)
+            g = torch.Generator().manual_seed(i)
+            bias = torch.randn(*shape, generator=g).to(bdt).to(gpu_device).requires_grad_(True)
+            ours = run_ours(q, k, v, do, bias, causal)
+            full = bias.detach().float().broadcast_to(B, H, Mc, N)
+            ref = run_oracle(q, k, v, do, full, causal)
+            assert ours["dbias"].shape == bias.shape and ours["dbias"].dtype == bdt
+            ref["dbias"] = ref["dbias"].sum_to_size((1,) * (4 - len(shape)) + tuple(shape)).reshape(shape)
+            check(ours, ref, "D%d %s %s causal=%s" % (D, bdt, shape, causal))
+
+
+def test_row_broadcast_bias_never_becomes_dense(gpu_device):
+    B, S, H, D = 1, 2048, 2, 16
+    q, k, v, do, _ = make_inputs(gpu_device, B, S, S, H, D, torch.bfloat16, None, seed=4)
+    bias = torch.randn(1, H, 1, S, generator=torch.Generator().manual_seed(4)).bfloat16().to(gpu_device).requires_grad_(True)
+    slopes = _slopes(H, gpu_device).requires_grad_(True)
+    dense_bytes = B * H * S * S * 2
+    for b in (bias, AlibiBias(slopes)):
+        torch.cuda.synchronize()
+        torch.cuda.reset_peak_memory_stats()
+        before = torch.cuda.memory_allocated()
+        ours = run_ours(q, k, v, do, b, False)
+        torch.cuda.synchronize()
+        assert torch.cuda.max_memory_allocated() - before < dense_bytes // 4
+        assert torch.isfinite(ours["dq"].float()).all()
+
+
+def test_batch_or_head_broadcast_bias(gpu_device):
+    """A bias broadcast over batches or heads only keeps its (M, N) tiles: read through an expanded
+    view, gradient computed densely and summed over the broadcast dimensions."""
+    B, M, N, H, D = 2, 200, 264, 3, 64
+    for i, shape in enumerate([(1, H, M, N), (B, 1, M, N), (1, 1, M, N), (M, N), (H, M, N)]):
+        q, k, v, do, _ = make_inputs(gpu_device, B, M, N, H, D, torch.float16, None, seed=60 + i)
+        g = torch.Generator().manual_seed(i)
+        bias = torch.randn(*shape, generator=g).bfloat16().to(gpu_device).requires_grad_(True)
+        ours = run_ours(q, k, v, do, bias, False)
+        ref = run_oracle(q, k, v, do, bias.detach().float().broadcast_to(B, H, M, N), False)
+        ref["dbias"] = ref["dbias"].sum_to_size((1,) * (4 - len(shape)) + tuple(shape)).reshape(shape)
+        check(ours, ref, str(shape))
+    # a bool mask of lower rank (key padding mask)
+    q, k, v, do, _ = make_inputs(gpu_device, B, M, N, H, D, torch.bfloat16, None, seed=70)
+    keep = torch.ones(B, 1, 1, N, dtype=torch.bool, device=gpu_device)
+    keep[0, ..., 200:] = False
+    keep[1, ..., 17:40] = False
+    check(run_ours(q, k, v, do, keep, False), run_oracle(q, k, v, do, keep.expand(B, H, M, N), False), "key padding")
+
+
+def test_reduced_gradient_without_allocations(gpu_device):
+    """The entry point that allocates nothing takes the column sums' partials from its static
+    array as well: same bits as the allocating one."""
+    B, M, N, H, D = 2, 256, 300, 4, 64
+    q, k, v, do, _ = make_inputs(gpu_device, B, M, N, H, D, torch.bfloat16, None, seed=90)
+    bias = torch.randn(1, H, 1, N, generator=torch.Generator().manual_seed(1)).bfloat16().to(gpu_device)
+    view = bias.expand(B, H, M, N)
+    o, lse = _flash_attn_fwd(q, k, v, view, False, D ** -0.5)
+    got = []
+    for noalloc in (False, True):
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        dbias = torch.full_like(bias, 7.0)
+        fa_mod._backend.bwd(do, q, k, v, o, view, False, D ** -0.5, lse, dq, dk, dv, dbias.expand(B, H, M, N), noalloc=noalloc)
+        torch.cuda.synchronize()
+        got.append((dq, dk, dv, dbias))
+    for a, b in zip(*got):
+        assert torch.isfinite(a.float()).all() and torch.equal(a, b)
+    slopes = _slopes(H, gpu_device)
+    got = []
+    for noalloc in (False, True):
+        dq, dk, dv, ds = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v), torch.full_like(slopes, 7.0)
+        o2, lse2 = _flash_attn_fwd(q, k, v, AlibiBias(slopes), False, D ** -0.5)
+        fa_mod._backend.bwd(do, q, k, v, o2, slopes, False, D ** -0.5, lse2, dq, dk, dv, ds, alibi=True, noalloc=noalloc)
+        torch.cuda.synchronize()
+        got.append((dq, dk, dv, ds))
+    for a, b in zip(*got):
+        assert torch.isfinite(a.float()).all() and torch.equal(a, b)
+
+
+# ---------------------------------------------------------------- V of another head dim, pruning
+def test_v_with_another_head_dim(gpu_device):
+    for d_qk, d_v, bias_kind, causal in [(64, 128, None, True), (128, 64, "bf16", False), (32, 64, "bool", False), (64, 16, None, False)]:
+        B, M, N, H = 2, 200, 200, 2
+        g = torch.Generator().manual_seed(d_qk + d_v)
+        mk = lambda *s: torch.randn(*s, generator=g).bfloat16().to(gpu_device)
+        q, k, v, do = mk(B, M, H, d_qk), mk(B, N, H, d_qk), mk(B, N, H, d_v), mk(B, M, H, d_v)
+        _, _, _, _, bias = make_inputs(gpu_device, B, M, N, H, 16, torch.bfloat16, bias_kind, seed=2)
+        ours = run_ours(q, k, v, do, bias, causal)
+        assert ours["out"].shape == (B, M, H, d_v) and ours["dv"].shape == v.shape and ours["dq"].shape == q.shape
+        check(ours, run_oracle(q, k, v, do, bias, causal), "Dqk%d Dv%d" % (d_qk, d_v))
+
+
+def test_gradients_nobody_asks_for_are_skipped(gpu_device):
+    """Only the kernels whose outputs are wanted run, and what they write equals the full run."""
+    B, M, N, H, D = 2, 300, 260, 2, 64
+    q, k, v, do, bias = make_inputs(gpu_device, B, M, N, H, D, torch.bfloat16, "bf16", seed=31)
+    full = run_ours(q, k, v, do, bias, False)
+    for wanted in [("q",), ("k", "v"), ("bias",), ("q", "bias"), ("v",)]:
+        t = {"q": q.detach().clone(), "k": k.detach().clone(), "v": v.detach().clone(), "bias": bias.detach().clone()}
+        for n in wanted:
+            t[n].requires_grad_(True)
+        flash_attention_fn(t["q"], t["k"], t["v"], t["bias"]).backward(do)
+        for n in ("q", "k", "v", "bias"):
+            if n in wanted:
+                assert torch.equal(t[n].grad, full["d" + n]), (wanted, n)
+            else:
+                assert t[n].grad is None
+
+
+# ---------------------------------------------------------------- the torch.library operator
+def test_library_operator_matches_the_function(gpu_device):
+    B, M, N, H, D = 1, 200, 200, 2, 64
+    q, k, v, do, bias = make_inputs(gpu_device, B, M, N, H, D, torch.bfloat16, "bf16", seed=41)
+    want = run_ours(q, k, v, do, bias, True)
+    q2, k2, v2 = (t.detach().clone().requires_grad_(True) for t in (q, k, v))
+    b2 = bias.detach().clone().requires_grad_(True)
+    out = flash_attention_op(q2, k2, v2, b2, True)
+    out.backward(do)
+    assert torch.equal(out, want["out"])
+    for got, n in ((q2.grad, "dq"), (k2.grad, "dk"), (v2.grad, "dv"), (b2.grad, "dbias")):
+        assert torch.equal(got, want[n]), n
+    torch.library.opcheck(torch.ops.fa_mi355.attention_fwd.default, (q, k, v, bias.detach(), True, 0.125),
+                          test_utils=("test_schema", "test_faketensor"))

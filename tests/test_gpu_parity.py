@@ -51,7 +51,7 @@ def run_ours(q, k, v, do, bias, causal, sm_scale=None):
     out = flash_attention_fn(q, k, v, bias, causal, sm_scale)
     out.backward(do)
     res = {"out": out.detach(), "dq": q.grad, "dk": k.grad, "dv": v.grad, "dbias": None}
-    if bias is not None and bias.requires_grad and bias.is_leaf:
+    if isinstance(bias, torch.Tensor) and bias.requires_grad and bias.is_leaf:
         res["dbias"] = bias.grad
         bias.grad = None
     return res

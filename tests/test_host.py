@@ -9,7 +9,7 @@ import pytest
 import torch
 
 import triton_flashattn_amd.flash_attention as fa_mod
-from triton_flashattn_amd import _native, flash_attention_fn, flash_attention_qkvpacked_fn
+from triton_flashattn_amd import AlibiBias, _native, flash_attention_fn, flash_attention_op, flash_attention_qkvpacked_fn
 from oracle.attention_oracle import attention_backward, attention_forward, reference_grads
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -23,20 +23,38 @@ class OracleBackend:
     def __init__(self):
         self.calls = []
 
-    def fwd(self, q, k, v, bias, causal, sm_scale, o, lse):
+    @staticmethod
+    def _alibi(slopes, M, N):
+        return AlibiBias(slopes).materialize(M, N)
+
+    def fwd(self, q, k, v, bias, causal, sm_scale, o, lse, alibi=False):
         self.calls.append(("fwd", q.stride(), None if bias is None else bias.stride()))
+        if alibi:
+            bias = self._alibi(bias, q.shape[1], k.shape[1])
         out, lse2 = attention_forward(q, k, v, bias, causal, sm_scale)
         o.copy_(out.to(o.dtype))
         lse.copy_(lse2)
 
-    def bwd(self, do, q, k, v, o, bias, causal, sm_scale, lse, dq, dk, dv, dbias, stages=7, workspace=None):
-        self.calls.append(("bwd", dq.stride(), dk.stride(), dv.stride()))
+    def bwd(self, do, q, k, v, o, bias, causal, sm_scale, lse, dq, dk, dv, dbias, stages=7, workspace=None,
+            noalloc=False, alibi=False):
+        self.calls.append(("bwd", None if dq is None else dq.stride(), None if dk is None else dk.stride(),
+                           None if dv is None else dv.stride(), stages))
+        slopes = bias
+        if alibi:
+            bias = self._alibi(bias, q.shape[1], k.shape[1])
         gq, gk, gv, gb, _ = attention_backward(do, q, k, v, o, lse, bias, causal, sm_scale)
-        dq.copy_(gq.to(dq.dtype))
-        dk.copy_(gk.to(dk.dtype))
-        dv.copy_(gv.to(dv.dtype))
-        if dbias is not None:
-            dbias.copy_(gb.to(dbias.dtype))
+        if dq is not None:
+            dq.copy_(gq.to(dq.dtype))
+        if dk is not None:
+            dk.copy_(gk.to(dk.dtype))
+            dv.copy_(gv.to(dv.dtype))
+        if dbias is not None and alibi:      # gradient of the slopes: dS . d bias / d slope
+            dist = self._alibi(torch.ones_like(slopes), q.shape[1], k.shape[1])
+            dbias.copy_((gb * dist).sum(dim=(0, 2, 3)))
+        elif dbias is not None:              # a view with zero strides along the reduced dimensions
+            red = [i for i in range(4) if dbias.stride(i) == 0 and dbias.shape[i] > 1]
+            g = gb.sum(dim=red, keepdim=True) if red else gb
+            dbias.as_strided(g.shape, dbias.stride()).copy_(g.to(dbias.dtype))
 
 
 @pytest.fixture
@@ -67,13 +85,19 @@ def test_rejects_bad_arguments(oracle_backend):
         flash_attention_fn(q, k[..., :8].repeat(1, 1, 1, 4), v)         # k head dim != q head dim (:775)
     q32, k32, v32 = _qkv(D=32)
     with pytest.raises(ValueError):
-        flash_attention_fn(q32, k32, v32[..., :16])                      # v head dim != q head dim
+        flash_attention_fn(q32, k32, v32[..., :8])                       # v head dim 8
     with pytest.raises(ValueError):
         flash_attention_fn(q, k[:, :, :1], v[:, :, :1])                  # head count
     with pytest.raises(ValueError):
         flash_attention_fn(q, k, v, causal=True)                         # causal with M != N (:777-778)
     with pytest.raises(ValueError):
-        flash_attention_fn(q, k, v, bias=torch.zeros(2, 1, 6, 9))        # bias not expanded to (B,H,M,N)
+        flash_attention_fn(q, k, v, bias=torch.zeros(2, 3, 6, 9))        # bias does not broadcast to (B,H,M,N)
+    with pytest.raises(ValueError):
+        flash_attention_fn(q, k, v, bias=torch.zeros(1, 2, 2, 6, 9))     # more than 4 dimensions
+    with pytest.raises(ValueError):
+        flash_attention_fn(q, k, v, bias=AlibiBias(torch.ones(3)))       # 3 slopes for 2 heads
+    with pytest.raises(TypeError):
+        AlibiBias(torch.ones(2, dtype=torch.float16))
     with pytest.raises(TypeError):
         flash_attention_fn(q, k, v, bias=torch.zeros(2, 2, 6, 9, dtype=torch.int32))
     with pytest.raises(ValueError):
@@ -160,6 +184,120 @@ def test_layout_normalisation(oracle_backend):
     assert oracle_backend.calls[-1][2] == (0, 0, 0, 1)
 
 
+# ---------------------------------------------------------------- beyond the reference's contract
+def test_broadcast_bias_and_reduced_gradient(oracle_backend):
+    """A bias with size-1 or missing leading dimensions is read through an expanded view; the
+    gradient of a row-broadcast bias reaches the backend as a view with zero strides (reduced in the
+    kernels), one broadcast over batches or heads only is computed densely and summed."""
+    B, M, N, H, D = 2, 6, 9, 2, 16
+    q, k, v = _qkv(B, M, N, H, D)
+    g = torch.Generator().manual_seed(11)
+    do = torch.randn(B, M, H, D, generator=g).bfloat16()
+    for shape in [(1, H, 1, N), (B, 1, 1, N), (N,), (H, M, N), (1, 1, M, N), (B, H, M, N)]:
+        bias = torch.randn(*shape, generator=g).bfloat16().requires_grad_(True)
+        out = flash_attention_fn(q, k, v, bias)
+        out.backward(do)
+        full = bias.detach().float().expand(B, H, M, N) if bias.dim() == 4 else bias.detach().float().broadcast_to(B, H, M, N)
+        ref = reference_grads(q, k, v, full, do)
+        assert torch.allclose(out.float(), ref["out"], atol=2e-2), shape
+        assert bias.grad.shape == bias.shape
+        want = ref["dbias"].sum_to_size(bias.shape if bias.dim() == 4 else (1,) * (4 - bias.dim()) + tuple(bias.shape))
+        assert torch.allclose(bias.grad.float().reshape(want.shape), want, atol=3e-2, rtol=3e-2), shape
+        fwd_call = [c for c in oracle_backend.calls if c[0] == "fwd"][-1]
+        assert all(st == 0 for st, n, w in zip(fwd_call[2], (1,) * (4 - bias.dim()) + tuple(shape), (B, H, M, N)) if n == 1 and w > 1)
+
+
+def test_alibi_bias_matches_materialized(oracle_backend):
+    B, M, N, H, D = 1, 8, 16, 4, 16
+    q, k, v = _qkv(B, M, N, H, D)
+    do = torch.randn(B, M, H, D, generator=torch.Generator().manual_seed(12)).bfloat16()
+    slopes = (2.0 ** (-8.0 * (torch.arange(H) + 1) / H)).float().requires_grad_(True)
+    q.requires_grad_(True)
+    out = flash_attention_fn(q, k, v, AlibiBias(slopes))
+    out.backward(do)
+    dense = AlibiBias(slopes.detach()).materialize(M, N).requires_grad_(True)
+    i, j = torch.arange(M)[:, None].float(), torch.arange(N)[None, :].float()
+    assert torch.equal(dense[0, 1], -slopes.detach()[1] * (i * N / M - j).abs())
+    ref = reference_grads(q, k, v, dense.detach(), do)
+    assert torch.allclose(out.float(), ref["out"], atol=2e-2)
+    dist = -(i * N / M - j).abs()
+    want = (ref["dbias"] * dist).sum(dim=(0, 2, 3))
+    assert slopes.grad.shape == (H,) and torch.allclose(slopes.grad, want, rtol=2e-2, atol=1e-3)  # o is bf16 in the stand-in
+    # packed entry
+    qkv = torch.randn(1, 8, 3, H, D).bfloat16().requires_grad_(True)
+    flash_attention_qkvpacked_fn(qkv, AlibiBias(slopes), True).sum().backward()
+    assert qkv.grad is not None
+
+
+def test_v_with_another_head_dim(oracle_backend):
+    g = torch.Generator().manual_seed(5)
+    B, M, N, H = 2, 6, 9, 2
+    for d_qk, d_v in ((16, 32), (64, 16)):
+        q = torch.randn(B, M, H, d_qk, generator=g).bfloat16().requires_grad_(True)
+        k = torch.randn(B, N, H, d_qk, generator=g).bfloat16().requires_grad_(True)
+        v = torch.randn(B, N, H, d_v, generator=g).bfloat16().requires_grad_(True)
+        do = torch.randn(B, M, H, d_v, generator=g).bfloat16()
+        out = flash_attention_fn(q, k, v)
+        assert out.shape == (B, M, H, d_v)
+        out.backward(do)
+        ref = reference_grads(q, k, v, None, do)          # sm_scale defaults to d_qk ** -0.5 on both sides
+        assert torch.allclose(out.float(), ref["out"], atol=2e-2)
+        for name, t in (("dq", q), ("dk", k), ("dv", v)):
+            assert t.grad.shape == t.shape
+            assert torch.allclose(t.grad.float(), ref[name], atol=3e-2, rtol=3e-2), (name, d_qk, d_v)
+
+
+def test_gradients_nobody_asks_for_are_not_computed(oracle_backend):
+    q, k, v = _qkv(M=8, N=8)
+    S = _native
+    q.requires_grad_(True)
+    flash_attention_fn(q, k, v).sum().backward()
+    assert oracle_backend.calls[-1][1] is not None and oracle_backend.calls[-1][2] is None      # dq only
+    assert oracle_backend.calls[-1][4] == S.FA_STAGE_PREP | S.FA_STAGE_DQ
+    q2, k2, v2 = _qkv(M=8, N=8)
+    v2.requires_grad_(True)
+    out = flash_attention_fn(q2, k2, v2)
+    out.sum().backward()
+    assert oracle_backend.calls[-1][1] is None and oracle_backend.calls[-1][4] == S.FA_STAGE_PREP | S.FA_STAGE_MAIN
+    assert v2.grad is not None and k2.grad is None
+    bias = torch.randn(2, 2, 8, 8).bfloat16().requires_grad_(True)
+    q3, k3, v3 = _qkv(M=8, N=8)
+    flash_attention_fn(q3, k3, v3, bias).sum().backward()     # only the bias wants a gradient
+    assert bias.grad is not None and oracle_backend.calls[-1][1] is None
+
+
+def test_autocast_casts_float32_inputs(oracle_backend, monkeypatch):
+    monkeypatch.setattr(torch, "is_autocast_enabled", lambda *a: True)
+    monkeypatch.setattr(torch, "get_autocast_dtype", lambda *a: torch.bfloat16)
+    q, k, v = (t.float() for t in _qkv())
+    out = flash_attention_fn(q, k, v)
+    assert out.dtype == torch.bfloat16
+
+
+def test_library_operator_traces_and_differentiates(oracle_backend):
+    q, k, v = _qkv(M=8, N=8)
+    bias = torch.randn(1, 2, 8, 8).bfloat16().requires_grad_(True)
+    q.requires_grad_(True)
+    out = flash_attention_op(q, k, v, bias, True)
+    out.float().pow(2).sum().backward()
+    ref = flash_attention_fn(q.detach(), k, v, bias.detach(), True)
+    assert torch.equal(out, ref) and q.grad is not None and bias.grad.shape == bias.shape
+    # fake-tensor implementations: shapes and dtypes without touching data
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    with FakeTensorMode():
+        fq, fk, fv = (torch.empty(2, 8, 2, 16, dtype=torch.bfloat16) for _ in range(3))
+        o, lse = torch.ops.fa_mi355.attention_fwd(fq, fk, fv, None, False, 0.25)
+        assert o.shape == (2, 8, 2, 16) and lse.shape == (2, 2, 8) and lse.dtype == torch.float32
+        grads = torch.ops.fa_mi355.attention_bwd(o, fq, fk, fv, o, lse, None, False, 0.25, False)
+        assert grads[0].shape == fq.shape and grads[3].numel() == 0
+
+
+def test_layout_rule_matches_the_c_side():
+    wide = torch.zeros(1, 4, 1, (1 << 23) + 16, dtype=torch.bfloat16)[..., :16]   # sequence stride >= 2^23 elements
+    assert not fa_mod._kernel_layout_ok(wide)
+    assert fa_mod._kernel_layout_ok(torch.zeros(1, 4, 1, 16, dtype=torch.bfloat16))
+
+
 # ---------------------------------------------------------------- C ABI surface (no launches)
 def _declared_functions():
     text = open(os.path.join(ROOT, "include", "fa_mi355.h")).read()
@@ -184,13 +322,13 @@ def test_struct_layouts_match_header():
 
 def test_abi_status_codes_and_workspace():
     lib = _native.load()
-    assert lib.fa_abi_version() == 1
+    assert lib.fa_abi_version() == 2
     assert lib.fa_strerror(0) == b"ok"
     assert b"head dimension" in lib.fa_strerror(-3)
     p = _native.FaProblem(B=2, H=3, M=100, N=50, D=64, dtype=_native.FA_BF16, bias_dtype=0, causal=0, sm_scale=0.1)
     rows = 2 * 3 * 100
     pad = lambda x: (x + 255) // 256 * 256
-    assert lib.fa_bwd_workspace_bytes(ctypes.byref(p)) == pad(rows * 4)
+    assert lib.fa_bwd_workspace_bytes(ctypes.byref(p)) == pad(rows * 4) + pad(2 * 3 * 50 * 4)   # delta + partial sums
     a = _native.FaFwdArgs()
     a.p = p
     assert lib.fa_fwd(ctypes.byref(a), None) == -1            # NULL pointers

@@ -7,10 +7,10 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libfa_mi355.so")
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 FA_F16, FA_BF16 = 0, 1
-FA_BIAS_NONE, FA_BIAS_BOOL, FA_BIAS_F16, FA_BIAS_BF16, FA_BIAS_F32 = 0, 1, 2, 3, 4
+FA_BIAS_NONE, FA_BIAS_BOOL, FA_BIAS_F16, FA_BIAS_BF16, FA_BIAS_F32, FA_BIAS_ALIBI = 0, 1, 2, 3, 4, 5
 
 _i64x4 = ctypes.c_int64 * 4
 

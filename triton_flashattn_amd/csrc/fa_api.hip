@@ -2,6 +2,9 @@
 // Host code only; the kernels live in fa_fwd.hip and fa_bwd.hip.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+#include <cstdio>
+#include <cstdlib>
 #include <mutex>
 
 #include "../../include/fa_mi355.h"
@@ -10,10 +13,10 @@
 namespace fa {
 // one object file per head dimension defines these (fa_fwd.hip, fa_bwd.hip with -DFA_HEAD_DIM)
 template <int D> hipError_t launch_fwd_d(const FwdParams& p, int dtype, int bias, bool causal, hipStream_t st);
-template <int D> hipError_t launch_bwd_d(const BwdParams& p, int dtype, int bias, bool causal, bool dbias, int stages, hipStream_t st);
+template <int D> hipError_t launch_bwd_d(const BwdParams& p, int dtype, int bias, bool causal, int dbias, int stages, hipStream_t st);
 #define FA_DECLARE_D(D)                                                                                         \
     template <> hipError_t launch_fwd_d<D>(const FwdParams& p, int dtype, int bias, bool causal, hipStream_t st); \
-    template <> hipError_t launch_bwd_d<D>(const BwdParams& p, int dtype, int bias, bool causal, bool dbias, int stages, hipStream_t st);
+    template <> hipError_t launch_bwd_d<D>(const BwdParams& p, int dtype, int bias, bool causal, int dbias, int stages, hipStream_t st);
 FA_DECLARE_D(16)
 FA_DECLARE_D(32)
 FA_DECLARE_D(64)
@@ -31,7 +34,7 @@ static hipError_t launch_fwd(const FwdParams& p, int D, int dtype, int bias, boo
     }
     return hipErrorNotSupported;
 }
-static hipError_t launch_bwd(const BwdParams& p, int D, int dtype, int bias, bool causal, bool dbias, int stages, hipStream_t st) {
+static hipError_t launch_bwd(const BwdParams& p, int D, int dtype, int bias, bool causal, int dbias, int stages, hipStream_t st) {
     switch (D) {
         case 16: return launch_bwd_d<16>(p, dtype, bias, causal, dbias, stages, st);
         case 32: return launch_bwd_d<32>(p, dtype, bias, causal, dbias, stages, st);
@@ -46,10 +49,11 @@ static int fwd_block_m() { return 128; }
 static int bwd_block_n(int) { return 128; }
 }  // namespace fa
 
-// Scratch of fa_bwd_noalloc: delta, one float per (batch, head, query row).  Every GPU the library
+// Scratch of fa_bwd_noalloc: delta, one float per (batch, head, query row), in the first half; the
+// partial sums of a reduced dbias in the second.  Every GPU the library
 // runs on holds its own copy of this array until the process ends.  In host code the name is only
 // a handle; the device address comes from hipGetSymbolAddress (scratch_on_current_device).
-static __device__ __align__(256) float scratch[FA_NOALLOC_MAX_ROWS];
+static __device__ __align__(256) float scratch[2 * FA_NOALLOC_MAX_ROWS];
 
 namespace fa {
 
@@ -82,7 +86,7 @@ int check_problem(const fa_problem& p) {
     if (p.B < 1 || p.H < 1 || p.M < 1 || p.N < 1) return FA_ERR_SHAPE;
     if (!head_dim_ok(p.D)) return FA_ERR_HEAD_DIM;
     if (p.dtype != FA_F16 && p.dtype != FA_BF16) return FA_ERR_DTYPE;
-    if (p.bias_dtype < FA_BIAS_NONE || p.bias_dtype > FA_BIAS_F32) return FA_ERR_DTYPE;
+    if (p.bias_dtype < FA_BIAS_NONE || p.bias_dtype > FA_BIAS_ALIBI) return FA_ERR_DTYPE;
     if (p.causal && p.M != p.N) return FA_ERR_SHAPE;
     // row indices times four (the LSE and delta vectors) are formed in 32 bits
     if (p.M >= (1 << 28) || p.N >= (1 << 28)) return FA_ERR_SHAPE;
@@ -134,6 +138,41 @@ bool bias_vec_ok(const void* ptr, const int64_t s[4], const fa_problem& p) {
 
 size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
+// With FA_MI355_VERBOSE set in the environment, says once per process on stderr when a bias cannot
+// take the 16-byte copy path and the kernels fall back to reading or writing it element by element
+// (much slower; the rules are in the header).
+void note_slow_bias(const char* what, const void* ptr, const int64_t s[4], const fa_problem& p) {
+    static std::atomic<bool> said{false};
+    if (!std::getenv("FA_MI355_VERBOSE") || said.exchange(true)) return;
+    std::fprintf(stderr,
+                 "libfa_mi355: %s takes the element-wise path (pointer %p, strides %lld/%lld/%lld/%lld elements, N = %d): "
+                 "needs unit key stride, 16-byte aligned base and B/H/M strides, rows of whole 16-byte chunks and "
+                 "(batch, head) slices below 2 GiB\n",
+                 what, ptr, (long long)s[0], (long long)s[1], (long long)s[2], (long long)s[3], p.N);
+}
+
+// the two parts of the backward scratch, in floats: delta, and the partial sums of a reduced
+// dbias (column sums per (batch, head, key), or slope gradients per (batch, head, key tile, wave))
+size_t delta_floats(const fa_problem& p) { return (size_t)p.B * p.H * p.M; }
+size_t partial_floats(const fa_problem& p) {
+    const size_t tiles4 = (size_t)((p.N + fa::bwd_block_n(p.D) - 1) / fa::bwd_block_n(p.D)) * 4;
+    return (size_t)p.B * p.H * ((size_t)p.N > tiles4 ? (size_t)p.N : tiles4);
+}
+
+// How dbias is laid out: 0 none, 1 dense (B, H, M, N), 2 reduced in the kernels; -1 = not acceptable
+int dbias_mode(const fa_bwd_args* a) {
+    const fa_problem& p = a->p;
+    if (!a->dbias) return 0;
+    if (p.bias_dtype == FA_BIAS_ALIBI) return 2;
+    const int64_t* s = a->dbias_strides;
+    const bool red_b = p.B > 1 && s[0] == 0, red_h = p.H > 1 && s[1] == 0, red_m = p.M > 1 && s[2] == 0;
+    if (!red_b && !red_h && !red_m) return 1;
+    // a reduction over batches or heads alone would need an (M, N) accumulator per output slice
+    if (!red_m && p.M > 1) return -1;
+    if (p.N > 1 && s[3] == 0) return -1;
+    return 2;
+}
+
 }  // namespace
 
 extern "C" {
@@ -147,11 +186,13 @@ const char* fa_strerror(int status) {
         case FA_ERR_SHAPE: return "bad shape: a dimension is < 1, too large, or causal with M != N";
         case FA_ERR_HEAD_DIM: return "head dimension must be one of 16, 32, 64, 128, 256";
         case FA_ERR_DTYPE: return "unsupported dtype / bias dtype (or dbias requested for a bool bias)";
-        case FA_ERR_LAYOUT: return "layout: head-dim stride must be 1 and pointers/strides 16-byte aligned";
+        case FA_ERR_LAYOUT:
+            return "layout: head-dim stride must be 1 and pointers/strides 16-byte aligned; a dbias broadcast over "
+                   "batches or heads must be broadcast over the query rows too";
         case FA_ERR_WORKSPACE: return "workspace is NULL, misaligned or smaller than fa_bwd_workspace_bytes()";
         case FA_ERR_UNSUPPORTED: return "combination not built into this library";
         case FA_ERR_LAUNCH: return "HIP kernel launch failed";
-        case FA_ERR_TOO_LARGE: return "fa_bwd_noalloc: B * H * M exceeds FA_NOALLOC_MAX_ROWS";
+        case FA_ERR_TOO_LARGE: return "fa_bwd_noalloc: the problem exceeds FA_NOALLOC_MAX_ROWS";
     }
     return "unknown status";
 }
@@ -172,9 +213,10 @@ int fa_fwd(const fa_fwd_args* a, void* stream) {
     k.sq = s3(a->q_strides); k.sk = s3(a->k_strides); k.sv = s3(a->v_strides); k.so = s3(a->o_strides);
     k.B = p.B; k.H = p.H; k.M = p.M; k.N = p.N;
     k.sm_scale = p.sm_scale;
-    if (a->bias) {
+    if (a->bias && p.bias_dtype != FA_BIAS_ALIBI) {
         k.sbias = s4(a->bias_strides);
         k.bias_vec = bias_vec_ok(a->bias, a->bias_strides, p) ? 1 : 0;
+        if (!k.bias_vec) note_slow_bias("bias", a->bias, a->bias_strides, p);
     }
     k.n_mtiles = (p.M + fa::fwd_block_m() - 1) / fa::fwd_block_m();
     hipError_t e = fa::launch_fwd(k, p.D, p.dtype, p.bias_dtype, p.causal != 0, static_cast<hipStream_t>(stream));
@@ -184,8 +226,7 @@ int fa_fwd(const fa_fwd_args* a, void* stream) {
 
 size_t fa_bwd_workspace_bytes(const fa_problem* p) {
     if (!p || check_problem(*p) != FA_OK) return 0;
-    size_t rows = (size_t)p->B * p->H * p->M;
-    return align256(rows * sizeof(float));
+    return align256(delta_floats(*p) * sizeof(float)) + align256(partial_floats(*p) * sizeof(float));
 }
 
 }  // extern "C"
@@ -200,34 +241,46 @@ int bwd_enqueue(const fa_bwd_args* a, void* stream, int stages, float* delta) {
     const fa_problem& p = a->p;
     int st = check_problem(p);
     if (st != FA_OK) return st;
-    if (!a->q || !a->k || !a->v || !a->o || !a->dout || !a->lse || !a->dq || !a->dk || !a->dv) return FA_ERR_NULL;
+    if (!a->q || !a->k || !a->v || !a->o || !a->dout || !a->lse) return FA_ERR_NULL;
+    // outputs of stages that do not run may be NULL
+    const bool need_dq = (stages & FA_STAGE_DQ) != 0, need_dkv = (stages & FA_STAGE_MAIN) != 0;
+    if ((need_dq && !a->dq) || (need_dkv && (!a->dk || !a->dv))) return FA_ERR_NULL;
     if ((p.bias_dtype != FA_BIAS_NONE) != (a->bias != nullptr)) return FA_ERR_NULL;
     if (a->dbias && (p.bias_dtype == FA_BIAS_NONE || p.bias_dtype == FA_BIAS_BOOL)) return FA_ERR_DTYPE;
+    const int db_mode = dbias_mode(a);
+    if (db_mode < 0) return FA_ERR_LAYOUT;
     if (!qkv_layout_ok(a->q, a->q_strides, p.B, p.M, p.H) || !qkv_layout_ok(a->k, a->k_strides, p.B, p.N, p.H) ||
         !qkv_layout_ok(a->v, a->v_strides, p.B, p.N, p.H) || !qkv_layout_ok(a->o, a->o_strides, p.B, p.M, p.H) ||
-        !qkv_layout_ok(a->dout, a->do_strides, p.B, p.M, p.H) || !qkv_layout_ok(a->dq, a->dq_strides, p.B, p.M, p.H) ||
-        !qkv_layout_ok(a->dk, a->dk_strides, p.B, p.N, p.H) || !qkv_layout_ok(a->dv, a->dv_strides, p.B, p.N, p.H))
+        !qkv_layout_ok(a->dout, a->do_strides, p.B, p.M, p.H) ||
+        (need_dq && !qkv_layout_ok(a->dq, a->dq_strides, p.B, p.M, p.H)) ||
+        (need_dkv && (!qkv_layout_ok(a->dk, a->dk_strides, p.B, p.N, p.H) || !qkv_layout_ok(a->dv, a->dv_strides, p.B, p.N, p.H))))
         return FA_ERR_LAYOUT;
+    float* partials = nullptr;
     if (!delta) {
         size_t need = fa_bwd_workspace_bytes(&p);
         if (!a->workspace || a->workspace_bytes < need || reinterpret_cast<uintptr_t>(a->workspace) % 256 != 0)
             return FA_ERR_WORKSPACE;
         delta = static_cast<float*>(a->workspace);
+        partials = reinterpret_cast<float*>(static_cast<char*>(a->workspace) + align256(delta_floats(p) * sizeof(float)));
+    } else {
+        partials = delta + FA_NOALLOC_MAX_ROWS;
     }
 
     fa::BwdParams k{};
     k.q = a->q; k.k = a->k; k.v = a->v; k.o = a->o; k.dout = a->dout; k.bias = a->bias; k.lse = a->lse;
     k.dq = a->dq; k.dk = a->dk; k.dv = a->dv; k.dbias = a->dbias;
     k.delta = delta;
+    k.partials = partials;
     k.sq = s3(a->q_strides); k.sk = s3(a->k_strides); k.sv = s3(a->v_strides); k.so = s3(a->o_strides);
     k.sdo = s3(a->do_strides); k.sdq = s3(a->dq_strides); k.sdk = s3(a->dk_strides); k.sdv = s3(a->dv_strides);
-    if (a->bias) {
+    if (a->bias && p.bias_dtype != FA_BIAS_ALIBI) {
         k.sbias = s4(a->bias_strides);
         k.bias_vec = bias_vec_ok(a->bias, a->bias_strides, p) ? 1 : 0;
     }
-    if (a->dbias) {
+    if (a->dbias && p.bias_dtype != FA_BIAS_ALIBI) {
         k.sdbias = s4(a->dbias_strides);
-        k.dbias_vec = bias_vec_ok(a->dbias, a->dbias_strides, p) ? 1 : 0;
+        k.dbias_vec = db_mode == 1 && bias_vec_ok(a->dbias, a->dbias_strides, p) ? 1 : 0;
+        if (db_mode == 1 && !k.dbias_vec) note_slow_bias("dbias", a->dbias, a->dbias_strides, p);
     }
     k.B = p.B; k.H = p.H; k.M = p.M; k.N = p.N;
     k.sm_scale = p.sm_scale;
@@ -235,7 +288,7 @@ int bwd_enqueue(const fa_bwd_args* a, void* stream, int stages, float* delta) {
     if (bn <= 0) return FA_ERR_UNSUPPORTED;
     k.n_ntiles = (p.N + bn - 1) / bn;
     k.n_mtiles = (p.M + fa::fwd_block_m() - 1) / fa::fwd_block_m();
-    hipError_t e = fa::launch_bwd(k, p.D, p.dtype, p.bias_dtype, p.causal != 0, a->dbias != nullptr, stages,
+    hipError_t e = fa::launch_bwd(k, p.D, p.dtype, p.bias_dtype, p.causal != 0, db_mode, stages,
                                   static_cast<hipStream_t>(stream));
     if (e == hipErrorNotSupported) return FA_ERR_UNSUPPORTED;
     return e == hipSuccess ? FA_OK : FA_ERR_LAUNCH;
@@ -253,7 +306,8 @@ int fa_bwd_noalloc(const fa_bwd_args* a, void* stream) {
     if (!a) return FA_ERR_NULL;
     int st = check_problem(a->p);
     if (st != FA_OK) return st;
-    if ((int64_t)a->p.B * a->p.H * a->p.M > (int64_t)FA_NOALLOC_MAX_ROWS) return FA_ERR_TOO_LARGE;
+    if (delta_floats(a->p) > (size_t)FA_NOALLOC_MAX_ROWS || partial_floats(a->p) > (size_t)FA_NOALLOC_MAX_ROWS)
+        return FA_ERR_TOO_LARGE;
     float* delta = fa::scratch_on_current_device();
     if (!delta) return FA_ERR_LAUNCH;
     return bwd_enqueue(a, stream, FA_STAGE_ALL, delta);

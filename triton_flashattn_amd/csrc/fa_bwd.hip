@@ -55,14 +55,15 @@ __global__ __launch_bounds__(256) void fa_bwd_prep_kernel(const BwdParams p) {
 // the bias ring instead of the bias, skips both recomputed products, the exponentials and the V
 // rows, and is one product instead of three.
 template <typename T, int D, int BIAS, bool CAUSAL, bool FROM_DS = false>
-__global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_dq_kernel(const BwdParams p) {
+__global__ __launch_bounds__(256, (StreamCfg<D, stream_kind(BIAS)>::MIN_BLOCKS)) void fa_bwd_dq_kernel(const BwdParams p) {
     static_assert(!FROM_DS || BIAS == 4 || (BIAS == 2 && __is_same(T, _Float16)) || (BIAS == 3 && __is_same(T, __bf16)),
                   "dS can stand in for the recomputation only in fp32 or in the element type of q");
-    typedef StreamCfg<D, BIAS> C;
+    constexpr int TB = tile_kind(BIAS);  // kind of bias tile that is streamed (none for ALiBi)
+    typedef StreamCfg<D, stream_kind(BIAS)> C;
     typedef Swz<D> SW;
     typedef typename VecOf<T>::v8 T8;
     typedef typename VecOf<T>::v4 T4;
-    typedef typename BiasElem<BIAS>::type E;
+    typedef typename BiasElem<tile_kind(BIAS)>::type E;
     constexpr int BM = C::BM, BK = C::BK, OS = C::OS, CPR = C::CPR;
 
     __shared__ __align__(1024) unsigned char smem[C::LDS_BYTES];
@@ -84,7 +85,12 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_
     const T* kp = reinterpret_cast<const T*>(p.k) + (int64_t)b * p.sk.b + (int64_t)h * p.sk.h;
     const T* vp = reinterpret_cast<const T*>(p.v) + (int64_t)b * p.sv.b + (int64_t)h * p.sv.h;
     const E* bp = nullptr;
-    if (BIAS != 0) bp = reinterpret_cast<const E*>(p.bias) + (int64_t)b * p.sbias.b + (int64_t)h * p.sbias.h;
+    if (TB != 0) bp = reinterpret_cast<const E*>(p.bias) + (int64_t)b * p.sbias.b + (int64_t)h * p.sbias.h;
+    float neg_slope = 0.f, ratio = 0.f;  // ALiBi: slope of this head, key positions per query row
+    if (BIAS == 5) {
+        neg_slope = -reinterpret_cast<const float*>(p.bias)[h];
+        ratio = (float)p.N / (float)p.M;
+    }
     if (FROM_DS) bp = reinterpret_cast<const E*>(p.dbias) + (int64_t)b * p.sdbias.b + (int64_t)h * p.sdbias.h;
 
     // Q^T and dO^T as B operands: column my_m, k = d
@@ -121,7 +127,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_
         for (int i = 0; i < 16; i++) dq_acc[db][i] = 0.f;
 
     const unsigned rows_l = SW::rows_lane(lane), cols_l = SW::cols_lane(lane);
-    KeyStream<T, D, BIAS, !FROM_DS> ks_;
+    KeyStream<T, D, stream_kind(BIAS), !FROM_DS> ks_;
     ks_.init(smem, kp, vp, bp, p.sk.s, p.sv.s, FROM_DS ? p.sdbias.m : p.sbias.m, FROM_DS ? p.sdbias.n : p.sbias.n, M, N,
              mw, wave, lane);
 
@@ -135,7 +141,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_
         ks_.template begin_step<BV>(k);
         const unsigned k_tile = ks_.k_addr(k), v_tile = ks_.v_addr(k);  // operand reads by address
         const unsigned char* b_lds = ks_.b_lds(k);
-        static_assert(BIAS == 0 || C::NH == 1, "a bias slot covers one 32-key block");
+        static_assert(TB == 0 || C::NH == 1, "a bias slot covers one 32-key block");
         // The step is consumed 32 keys at a time, so that only one 32 x 32 score block is live.
 #pragma unroll
         for (int nb = 0; nb < C::NH; nb++) {
@@ -215,6 +221,10 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_
                         f32x4 w = *reinterpret_cast<const f32x4*>(b_lds + ks_.b_off(r, nl));
 #pragma unroll
                         for (int e = 0; e < 4; e++) bv[e] = w[e];
+                    } else if constexpr (BIAS == 5) {
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            bv[e] = alibi_bias(neg_slope, ratio, (float)my_m, (float)(n0 + nh + 4 * g) + (float)(8 * q4 + e));
                     }
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
@@ -276,7 +286,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_bwd_
 #pragma unroll 1
         for (int k = n_fast; k < n_steps; k++) kv_step(k, std::true_type{}, bv_tag);
     };
-    if (FROM_DS || (BIAS != 0 && p.bias_vec)) run(std::true_type{});
+    if (FROM_DS || (TB != 0 && p.bias_vec)) run(std::true_type{});
     else run(std::false_type{});
 
     // ---- epilogue: dq = dQ * sm_scale (flash_attention.py:644-646) ----
@@ -331,6 +341,10 @@ template <> struct BiasQuad<3> {
         raw = lds_read_tr4(reinterpret_cast<const __bf16*>(slice) + tr_offset(lane, row0, 0, 32));
     }
     __device__ __forceinline__ float get(int e) const { return (float)__builtin_bit_cast(bf16x4, raw)[e]; }
+};
+template <> struct BiasQuad<5> {  // ALiBi: nothing to read, the kernel computes the term from the indices
+    __device__ __forceinline__ void load(const unsigned char*, int, int, int) {}
+    __device__ __forceinline__ float get(int) const { return 0.f; }
 };
 template <> struct BiasQuad<4> {
     float v[4];
@@ -397,16 +411,21 @@ template <int D, int BIAS> struct BwdCfg {
 //   step t : S-wave : P(t+1) from Q(t+1), then dV += dO(t)^T P(t)        (P(t) kept in registers)
 //            dP-wave: dS(t) from dO(t) and the P(t) handed over in step t-1, dK += Q(t-1)^T dS(t-1)
 // While one wave of a SIMD runs exponentials or products the other issues MFMAs.
-template <typename T, int D, int BIAS, bool CAUSAL, bool DBIAS>
+// DBIAS: 0 = the bias is not trainable; 1 = dBias is written densely, (B, H, M, N) in the bias dtype
+// (flash_attention.py:307-308); 2 = reduced in the kernel: for a float bias the sums of dS over the
+// query rows, one fp32 per (batch, head, key), for ALiBi the gradient of the slope, one fp32 per
+// (batch, head, key tile, wave); a second small kernel sums those over the broadcast dimensions.
+template <typename T, int D, int BIAS, bool CAUSAL, int DBIAS>
 __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
-    typedef BwdCfg<D, BIAS> C;
+    constexpr int TB = tile_kind(BIAS);  // kind of bias tile that is streamed (none for ALiBi)
+    typedef BwdCfg<D, TB> C;
     typedef Swz<D> SW;
     typedef typename VecOf<T>::v8 T8;
     typedef typename VecOf<T>::v4 T4;
-    typedef typename BiasElem<BIAS>::type E;
+    typedef typename BiasElem<tile_kind(BIAS)>::type E;
     constexpr int BN = C::BN, BMI = C::BMI, CPR = C::CPR, DSS = C::DSS, NSUB = C::NSUB;
     // dBias leaves through the dS tile (16-byte row stores) when it has the element type of dS
-    constexpr bool DB_VIA_LDS = DBIAS && ((BIAS == 2 && __is_same(T, _Float16)) || (BIAS == 3 && __is_same(T, __bf16)));
+    constexpr bool DB_VIA_LDS = DBIAS == 1 && ((BIAS == 2 && __is_same(T, _Float16)) || (BIAS == 3 && __is_same(T, __bf16)));
 
     __shared__ __align__(16) unsigned char smem[C::LDS_BYTES];
 
@@ -433,8 +452,13 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
     const float* deltap = p.delta + ((int64_t)b * p.H + h) * M;
     const E* bp = nullptr;
     E* dbp = nullptr;
-    if (BIAS != 0) bp = reinterpret_cast<const E*>(p.bias) + (int64_t)b * p.sbias.b + (int64_t)h * p.sbias.h;
-    if (DBIAS) dbp = reinterpret_cast<E*>(p.dbias) + (int64_t)b * p.sdbias.b + (int64_t)h * p.sdbias.h;
+    if (TB != 0) bp = reinterpret_cast<const E*>(p.bias) + (int64_t)b * p.sbias.b + (int64_t)h * p.sbias.h;
+    if (DBIAS == 1) dbp = reinterpret_cast<E*>(p.dbias) + (int64_t)b * p.sdbias.b + (int64_t)h * p.sdbias.h;
+    float neg_slope = 0.f, ratio = 0.f;  // ALiBi: slope of this head, key positions per query row
+    if (BIAS == 5) {
+        neg_slope = -reinterpret_cast<const float*>(p.bias)[h];
+        ratio = (float)p.N / (float)p.M;
+    }
     unsigned char* ring_lds = smem + C::OFF_BIAS + kb * C::RING * C::BT_BYTES;
     float* p_lds = reinterpret_cast<float*>(smem + C::OFF_P) + kb * NSUB * 64 * 16;  // + buffer * P_BYTES / 4
 
@@ -461,11 +485,11 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
     const int n_mblocks = (M + BMI - 1) / BMI;
     // causal: query blocks that end above the first key of this tile see none of its keys
     const int mb_first = CAUSAL ? (n0 / BMI) : 0;
-    const bool bias_vec = BIAS != 0 && p.bias_vec;
-    const bool dbias_vec = DBIAS && p.dbias_vec;
+    const bool bias_vec = TB != 0 && p.bias_vec;
+    const bool dbias_vec = DBIAS == 1 && p.dbias_vec;
 
     // blocks skipped by the causal schedule still owe zeros to dBias
-    if (DBIAS && CAUSAL && !s_wave) {
+    if (DBIAS == 1 && CAUSAL && !s_wave) {
         const int rows_skipped = mb_first * BMI < M ? mb_first * BMI : M;
         for (int c = lane; c < rows_skipped * C::BCPR; c += 64) {
             const int m = c / C::BCPR, nn = nw + (c % C::BCPR) * C::EPC;
@@ -527,7 +551,7 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
     // is the row-major slice.  Rows past M re-read row M - 1 and chunks that start past N re-read
     // column 0: both are masked where they are used.
     auto issue_bias = [&](int mb) {
-        if constexpr (BIAS != 0) {
+        if constexpr (TB != 0) {
             const unsigned dst = lds_base + C::OFF_BIAS + (kb * C::RING + (mb - mb_first) % C::RING) * C::BT_BYTES;
             const uint64_t base = uniform_ptr(bp);
 #pragma unroll
@@ -558,7 +582,7 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
     constexpr bool Q_BY_S = true, DO_BY_S = false;
     // per-element path for bias rows that cannot be copied in aligned 16-byte chunks
     auto load_bias_scalar = [&](int mb, unsigned char* dst) {
-        if constexpr (BIAS != 0) {
+        if constexpr (TB != 0) {
             const int m0 = mb * BMI;
 #pragma unroll 1
             for (int row = g; row < BMI; row += 2) {
@@ -576,7 +600,7 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
 #pragma unroll 1
         for (int i = 0; i < C::LA; i++) {
             if (s_wave == Q_BY_S) issue_q(mb_first + i);
-            if (s_wave && BIAS != 0 && bias_vec) issue_bias(mb_first + i);
+            if (s_wave && TB != 0 && bias_vec) issue_bias(mb_first + i);
             if (s_wave == DO_BY_S && i < C::LA - 1) issue_do(mb_first + i);
         }
         lds_copy_end(saved_m0);
@@ -653,7 +677,7 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
         // while the partner does its vector work.  It needs the Q block one step earlier, i.e. a copy
         // look-ahead of at least three blocks.  Measured: 6 % on the kernel with a bias (where the
         // vector work is heaviest), a loss of 4 % without one, which keeps the plain order.
-        constexpr bool S_AHEAD = BIAS != 0 && C::LA >= 3;
+        constexpr bool S_AHEAD = TB != 0 && C::LA >= 3;
         f32x16 sacc[NSUB];
         if constexpr (S_AHEAD) {
             T8 a_rows[NR];
@@ -695,6 +719,7 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
             auto make_p = [&]() {
                 const int m0 = nb * BMI;
                 const bool need_mask = (m0 + BMI > M) || (n0 + BN > N) || (CAUSAL && m0 < n0 + BN - 1);
+                const float mf0 = (float)(m0 + 4 * g);  // ALiBi: first row of this lane's registers, as a float
                 float* p_out = p_lds + (nb & 1) * (C::P_BYTES / 4);
                 auto p_step = [&](auto masked_tag) {
                     constexpr bool MASKED = decltype(masked_tag)::value;
@@ -709,7 +734,8 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
                             for (int e = 0; e < 4; e++) {
                                 const int i = q4 * 4 + e;
                                 // bool mask: the additive term in log2 units; float bias: natural units
-                                const float bv = bias_in[sb][q4].get(e);
+                                float bv = bias_in[sb][q4].get(e);
+                                if constexpr (BIAS == 5) bv = alibi_bias(neg_slope, ratio, mf0 + (float)(ml0 - 4 * g + e), (float)my_n);
                                 float pv;
                                 if constexpr (MASKED) {
                                     const int m = m0 + ml0 + e;
@@ -718,7 +744,7 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
                                     float tmask = oob ? kMask : 0.f;
                                     if (CAUSAL) tmask += (m < my_n) ? kMask : 0.f;
                                     float add = BIAS >= 2 ? __fmul_rn(bv, kLog2e) : bv;
-                                    if (BIAS != 0) add = oob ? kMask : add;
+                                    if (BIAS != 0) add = oob ? kMask : add;  // out-of-range bias reads as masked
                                     x = __fadd_rn(x, __fadd_rn(tmask, add));
                                     pv = fast_exp2(x - lse4[e]);
                                 } else {
@@ -736,7 +762,7 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
                 if (need_mask) p_step(std::true_type{});
                 else p_step(std::false_type{});
             };
-            if constexpr (BIAS != 0 && !BV) {
+            if constexpr (TB != 0 && !BV) {
                 if (nb < n_mblocks) load_bias_scalar(nb, ring_lds + ((nb - mb_first) % C::RING) * C::BT_BYTES);
             }
             if constexpr (S_AHEAD) {
@@ -758,14 +784,14 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
                 if (nb + 1 < n_mblocks) mma_rows(a_rows, sacc);
             } else {
                 T8 a_cols[NA], a_rows[NR];
-                if constexpr (BIAS == 0) issue_copies();
+                if constexpr (TB == 0) issue_copies();
                 load_cols(do_tile(t), a_cols);
                 load_rows(q_tile(nb), a_rows);
                 if constexpr (PRELOAD) {
                     load_p_inputs();
                     __builtin_amdgcn_sched_barrier(0);
                 }
-                if constexpr (BIAS != 0) issue_copies();
+                if constexpr (TB != 0) issue_copies();
                 // dV^T += dO(t)^T P(t) first: its operands do not depend on this step
                 if (t >= mb_first && t < n_mblocks) mma_cols(a_cols, op_cur);
                 if (nb < n_mblocks) {
@@ -789,7 +815,7 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
 #pragma unroll 1
         for (int t = mb_first - 1; t <= n_mblocks; t++) s_step(t);
         };
-        if (BIAS != 0 && bias_vec) s_loop(std::true_type{});
+        if (TB != 0 && bias_vec) s_loop(std::true_type{});
         else s_loop(std::false_type{});
     } else {
         // ================================ dP-wave ================================
@@ -815,6 +841,7 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
                 db_off[it] = nn < N ? db_row * db_row_bytes + nn * 2 : (int)0x80000000;
             }
         }
+        float red_acc = 0.f;  // DBIAS == 2: this lane's share of the reduced gradient
         auto dp_loop = [&](auto fast_tag) {
         constexpr bool DB_FAST = decltype(fast_tag)::value;
         // copies per step; the dBias stores that may sit between them in the queue are not
@@ -845,12 +872,12 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
                         p_vals[sb][q4] = *reinterpret_cast<const f32x4*>(p_in + ((sb * 4 + q4) * 64 + lane) * 4);
                     }
             };
-            if constexpr (BIAS == 0) issue_copies();
+            if constexpr (TB == 0) issue_copies();
             // operands of both products up front: Q(t-1)^T for dK, the rows of dO(t) for dP
             if constexpr (C::DEFER_DK) load_cols(q_tile(t - 1), a_cols);
             load_rows(do_tile(t), a_rows);
-            if constexpr (PRELOAD && BIAS == 0) __builtin_amdgcn_sched_barrier(0);
-            if constexpr (BIAS != 0) issue_copies();  // behind the reads, whose round trip they cover
+            if constexpr (PRELOAD && TB == 0) __builtin_amdgcn_sched_barrier(0);
+            if constexpr (TB != 0) issue_copies();  // behind the reads, whose round trip they cover
             if (C::DEFER_DK && t - 1 >= mb_first) mma_cols(a_cols, op_cur);  // dK^T += Q(t-1)^T dS(t-1)
             if (live) {
                 f32x16 sacc[NSUB];
@@ -875,7 +902,13 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
                             const float dsv = p4[e] * (sacc[sb][i] - del4[e]);
                             op_cur[sb][i >> 3][i & 7] = (T)dsv;
                             d4[e] = (T)dsv;
-                            if constexpr (DBIAS && !DB_VIA_LDS) {
+                            if constexpr (DBIAS == 2) {
+                                // rows past M and keys past N have P = 0 exactly, hence dS = 0
+                                if constexpr (BIAS == 5)  // d bias / d slope = -|i N / M - j|
+                                    red_acc -= dsv * __builtin_fabsf(__builtin_fmaf((float)(m0 + 4 * g) + (float)(ml0 - 4 * g + e), ratio, -(float)my_n));
+                                else red_acc += dsv;
+                            }
+                            if constexpr (DBIAS == 1 && !DB_VIA_LDS) {
                                 const int m = m0 + ml0 + e;
                                 if (m < M && my_n < N) dbp[(int64_t)m * p.sdbias.m + (int64_t)my_n * p.sdbias.n] = (E)dsv;
                             }
@@ -925,6 +958,20 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
         } else {
             dp_loop(std::false_type{});
         }
+        if constexpr (DBIAS == 2) {
+            if constexpr (BIAS == 5) {
+                // slope gradient of this wave's 32 keys: one float per (batch, head, key tile, wave), summed
+                // over the lanes in a fixed order
+                float s = red_acc;
+#pragma unroll
+                for (int w = 32; w >= 1; w >>= 1) s += __shfl_xor(s, w, 64);
+                if (lane == 0) p.partials[((int64_t)bh * p.n_ntiles + nt) * 4 + kb] = s;
+            } else {
+                // column sums: lanes l and l + 32 hold different rows of the same key
+                const float s = pair_sum(red_acc);
+                if (g == 0 && my_n < N) p.partials[(int64_t)bh * N + my_n] = s;
+            }
+        }
     }
     // ---- dV (S-wave) or dK (dP-wave) of this wave's 32 keys (flash_attention.py:449-454) ----
     if (my_n < N) {
@@ -948,14 +995,47 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
 }
 
 // ---------------------------------------------------------------------------------------------
-template <typename T, int D, int BIAS, bool CAUSAL, bool DBIAS>
+template <typename T, int D, int BIAS, bool CAUSAL, int DBIAS>
 static hipError_t launch_main(const BwdParams& p, hipStream_t st) {
     dim3 grid((unsigned)(p.n_ntiles * p.B * p.H));
     hipLaunchKernelGGL((fa_bwd_kernel<T, D, BIAS, CAUSAL, DBIAS>), grid, dim3(512), 0, st, p);
     return hipGetLastError();
 }
 
-template <typename T, int D> static hipError_t launch_all(const BwdParams& p, int bias, bool causal, bool dbias, int stages, hipStream_t st) {
+// ---------------------------------------------------------------------------------------------
+// Second pass of the reduced dBias modes (DBIAS == 2), one thread per output element, sums in a
+// fixed order: every output has one writer and the result is reproducible run to run.
+//   float bias: dbias[b', h', 0, n] = sum over the broadcast batches / heads of colsum[b, h, n]
+template <typename E>
+__global__ __launch_bounds__(256) void fa_bwd_colsum_reduce_kernel(const BwdParams p) {
+    const int nb_out = p.sdbias.b == 0 ? 1 : p.B, nh_out = p.sdbias.h == 0 ? 1 : p.H;
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (int64_t)nb_out * nh_out * p.N) return;
+    const int n = (int)(idx % p.N);
+    const int ho = (int)((idx / p.N) % nh_out), bo = (int)(idx / ((int64_t)p.N * nh_out));
+    float s = 0.f;
+    for (int b = (nb_out == 1 ? 0 : bo); b < (nb_out == 1 ? p.B : bo + 1); b++)
+        for (int h = (nh_out == 1 ? 0 : ho); h < (nh_out == 1 ? p.H : ho + 1); h++)
+            s += p.partials[((int64_t)b * p.H + h) * p.N + n];
+    reinterpret_cast<E*>(p.dbias)[(int64_t)bo * p.sdbias.b + (int64_t)ho * p.sdbias.h + (int64_t)n * p.sdbias.n] = (E)s;
+}
+//   ALiBi: dslope[h] = sum over batches, key tiles and waves of the partial slope gradients
+// (a template so that the per-head-dim compile units may each hold a copy)
+template <int LANES>
+__global__ __launch_bounds__(LANES) void fa_bwd_slope_reduce_kernel(const BwdParams p) {
+    static_assert(LANES == 64, "one wave");
+    const int h = blockIdx.x, lane = threadIdx.x;
+    const int per_bh = p.n_ntiles * 4;
+    float s = 0.f;
+    for (int b = 0; b < p.B; b++)
+        for (int i = lane; i < per_bh; i += 64) s += p.partials[((int64_t)b * p.H + h) * per_bh + i];
+#pragma unroll
+    for (int w = 32; w >= 1; w >>= 1) s += __shfl_xor(s, w, 64);
+    if (lane == 0) reinterpret_cast<float*>(p.dbias)[h] = s;
+}
+
+// dbias: 0 = none, 1 = dense, 2 = reduced in the kernels (see fa_bwd_kernel)
+template <typename T, int D> static hipError_t launch_all(const BwdParams& p, int bias, bool causal, int dbias, int stages, hipStream_t st) {
     constexpr int RPB = 256 / (D / 8);
     const int64_t rows = (int64_t)p.B * p.H * p.M;
     dim3 rgrid((unsigned)((rows + RPB - 1) / RPB));
@@ -969,31 +1049,49 @@ template <typename T, int D> static hipError_t launch_all(const BwdParams& p, in
 #define FA_CASE(BK, DBK)                                                                                      \
     if (bias == BK && dbias == DBK)                                                                           \
         e = causal ? launch_main<T, D, BK, true, DBK>(p, st) : launch_main<T, D, BK, false, DBK>(p, st);
-    FA_CASE(0, false)
-    else FA_CASE(1, false)
-    else FA_CASE(2, false)
-    else FA_CASE(2, true)
-    else FA_CASE(3, false)
-    else FA_CASE(3, true)
-    else FA_CASE(4, false)
-    else FA_CASE(4, true)
+    FA_CASE(0, 0)
+    else FA_CASE(1, 0)
+    else FA_CASE(2, 0)
+    else FA_CASE(2, 1)
+    else FA_CASE(2, 2)
+    else FA_CASE(3, 0)
+    else FA_CASE(3, 1)
+    else FA_CASE(3, 2)
+    else FA_CASE(4, 0)
+    else FA_CASE(4, 1)
+    else FA_CASE(4, 2)
+    else FA_CASE(5, 0)
+    else FA_CASE(5, 2)
     else return hipErrorInvalidValue;
 #undef FA_CASE
         if (e != hipSuccess) return e;
+        if (dbias == 2) {
+            if (bias == 5) {
+                hipLaunchKernelGGL((fa_bwd_slope_reduce_kernel<64>), dim3((unsigned)p.H), dim3(64), 0, st, p);
+            } else {
+                const int64_t outs = (int64_t)(p.sdbias.b == 0 ? 1 : p.B) * (p.sdbias.h == 0 ? 1 : p.H) * p.N;
+                dim3 g((unsigned)((outs + 255) / 256));
+                if (bias == 2) hipLaunchKernelGGL((fa_bwd_colsum_reduce_kernel<_Float16>), g, dim3(256), 0, st, p);
+                else if (bias == 3) hipLaunchKernelGGL((fa_bwd_colsum_reduce_kernel<__bf16>), g, dim3(256), 0, st, p);
+                else hipLaunchKernelGGL((fa_bwd_colsum_reduce_kernel<float>), g, dim3(256), 0, st, p);
+            }
+            e = hipGetLastError();
+            if (e != hipSuccess) return e;
+        }
     }
     if (stages & 4) {
         dim3 qgrid((unsigned)(p.n_mtiles * p.B * p.H));
-        // dBias in fp32 or in the element type of q, written a moment ago by the key-tile kernel in
-        // rows of whole 16-byte chunks, is the dS the dQ product needs.  Only when that kernel ran in
+        // dBias in fp32 or in the element type of q, written densely a moment ago by the key-tile kernel
+        // in rows of whole 16-byte chunks, is the dS the dQ product needs.  Only when that kernel ran in
         // this very call (or the caller vouches for the contents of dbias, bit 8) is it read.
         constexpr int DS_BIAS = __is_same(T, _Float16) ? 2 : 3;
-        const bool ds_valid = (stages & 2) || (stages & 8);
-        if (ds_valid && dbias && bias == DS_BIAS && p.dbias_vec) {
+        const bool ds_valid = dbias == 1 && ((stages & 2) || (stages & 8));
+        if (ds_valid && bias == DS_BIAS && p.dbias_vec) {
             if (causal) hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, DS_BIAS, true, true>), qgrid, dim3(256), 0, st, p);
             else hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, DS_BIAS, false, true>), qgrid, dim3(256), 0, st, p);
             return hipGetLastError();
         }
-        if (ds_valid && dbias && bias == 4 && p.dbias_vec) {
+        if (ds_valid && bias == 4 && p.dbias_vec) {
             if (causal) hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, 4, true, true>), qgrid, dim3(256), 0, st, p);
             else hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, 4, false, true>), qgrid, dim3(256), 0, st, p);
             return hipGetLastError();
@@ -1009,6 +1107,7 @@ template <typename T, int D> static hipError_t launch_all(const BwdParams& p, in
             FA_CASE(2)
             FA_CASE(3)
             FA_CASE(4)
+            FA_CASE(5)
             default: return hipErrorInvalidValue;
         }
 #undef FA_CASE
@@ -1022,8 +1121,8 @@ template <typename T, int D> static hipError_t launch_all(const BwdParams& p, in
 #ifndef FA_HEAD_DIM
 #error "compile with -DFA_HEAD_DIM=<16|32|64|128|256>"
 #endif
-template <int D> hipError_t launch_bwd_d(const BwdParams& p, int dtype, int bias, bool causal, bool dbias, int stages, hipStream_t st);
-template <> hipError_t launch_bwd_d<FA_HEAD_DIM>(const BwdParams& p, int dtype, int bias, bool causal, bool dbias, int stages, hipStream_t st) {
+template <int D> hipError_t launch_bwd_d(const BwdParams& p, int dtype, int bias, bool causal, int dbias, int stages, hipStream_t st);
+template <> hipError_t launch_bwd_d<FA_HEAD_DIM>(const BwdParams& p, int dtype, int bias, bool causal, int dbias, int stages, hipStream_t st) {
     if (dtype == 0) return launch_all<_Float16, FA_HEAD_DIM>(p, bias, causal, dbias, stages, st);
     return launch_all<__bf16, FA_HEAD_DIM>(p, bias, causal, dbias, stages, st);
 }

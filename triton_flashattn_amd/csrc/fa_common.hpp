@@ -249,6 +249,21 @@ template <> struct BiasElem<1> { typedef unsigned char type; };
 template <> struct BiasElem<2> { typedef _Float16 type; };
 template <> struct BiasElem<3> { typedef __bf16 type; };
 template <> struct BiasElem<4> { typedef float type; };
+template <> struct BiasElem<5> { typedef float type; };  // ALiBi: one fp32 slope per head, no tile
+template <> struct BiasElem<6> { typedef unsigned char type; };  // the stream kind of ALiBi (below)
+
+// Bias kind 5 (ALiBi): bias[b,h,i,j] = -slope[h] * |i * N / M - j| is computed from the indices, so no
+// bias tile exists and the K/V stream is tiled as without a bias.  TILE_KIND maps a bias kind to
+// the kind of tile that StreamCfg / KeyStream handle.
+constexpr int tile_kind(int bias) { return bias == 5 ? 0 : bias; }
+// ... and to the kind that StreamCfg / KeyStream tile the K/V stream for: 6 = no bias tile, but steps of
+// 32 keys like the kernels with one (the element-wise work of ALiBi needs the registers that the
+// 64-key steps of the bias-free kernels spend on a second block of scores)
+constexpr int stream_kind(int bias) { return bias == 5 ? 6 : bias; }
+// -slope * |m * ratio - n| for query row m and key n (both exact as floats), natural units
+__device__ __forceinline__ float alibi_bias(float neg_slope, float ratio, float mf, float nf) {
+    return neg_slope * __builtin_fabsf(__builtin_fmaf(mf, ratio, -nf));
+}
 
 // Tiling of the forward and the dQ kernel: a work-group owns 128 query rows (4 waves x 32 rows) and streams
 // keys in steps of NH blocks of 32.  K and V rows of a step and the bias slice of each wave reach
@@ -265,7 +280,7 @@ template <int D, int BIAS> struct StreamCfg {
     static constexpr int CPR = D / 8;                // 16-byte chunks per row
     static constexpr int KSTEPS = D / 16;            // MFMA k-steps of Q K^T
     static constexpr int DB = DP / 32;               // 32-wide blocks of the head dim
-    static constexpr int ES = BIAS == 0 ? 0 : (BIAS == 1 ? 1 : (BIAS == 4 ? 4 : 2));
+    static constexpr int ES = (BIAS == 0 || BIAS == 6) ? 0 : (BIAS == 1 ? 1 : (BIAS == 4 ? 4 : 2));
     static constexpr int EPC = ES > 0 ? 16 / ES : 8; // bias elements per 16-byte chunk
     static constexpr int STEP_BYTES = BK * D * 2;    // K (or V) rows of one step, unpadded, swizzled
     static constexpr int NKD = STEP_BYTES / 1024;    // 1 KB copies per K (or V) step
@@ -370,7 +385,7 @@ template <typename T, int D, int BIAS, bool WITH_V = true> struct KeyStream {
     // of the row.  Rows past M re-read row M - 1 (never stored) and chunks that start past N
     // re-read column 0 (masked).
     __device__ __forceinline__ void issue_bias(int k) {
-        if constexpr (BIAS != 0) {
+        if constexpr (C::ES != 0) {
             const unsigned dst = lds_bias + (k % C::NBS) * C::BSLOT;
             const uint64_t base = uniform_ptr(bp);
 #pragma unroll
@@ -410,7 +425,7 @@ template <typename T, int D, int BIAS, bool WITH_V = true> struct KeyStream {
         // the copies of the steps since may still be in flight
         wait_vmcnt<(BV ? C::BCH : 0) + OPS*(C::LA - 1)>();
         lds_barrier();
-        if constexpr (BIAS != 0 && !BV) {
+        if constexpr (C::ES != 0 && !BV) {
             // unaligned bias rows or non-unit key stride: one element per lane per row
             if (lane < 32) {
 #pragma unroll 1

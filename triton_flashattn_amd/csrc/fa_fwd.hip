@@ -27,12 +27,13 @@
 namespace fa {
 
 template <typename T, int D, int BIAS, bool CAUSAL>
-__global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_kernel(const FwdParams p) {
-    typedef StreamCfg<D, BIAS> C;
+__global__ __launch_bounds__(256, (StreamCfg<D, stream_kind(BIAS)>::MIN_BLOCKS)) void fa_fwd_kernel(const FwdParams p) {
+    constexpr int TB = tile_kind(BIAS);  // kind of bias tile that is streamed (none for ALiBi)
+    typedef StreamCfg<D, stream_kind(BIAS)> C;
     typedef Swz<D> SW;
     typedef typename VecOf<T>::v8 T8;
     typedef typename VecOf<T>::v4 T4;
-    typedef typename BiasElem<BIAS>::type E;
+    typedef typename BiasElem<tile_kind(BIAS)>::type E;
     constexpr int BM = C::BM, BK = C::BK, OS = C::OS, CPR = C::CPR;
 
     __shared__ __align__(1024) unsigned char smem[C::LDS_BYTES];
@@ -54,7 +55,13 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_
     const T* kp = reinterpret_cast<const T*>(p.k) + (int64_t)b * p.sk.b + (int64_t)h * p.sk.h;
     const T* vp = reinterpret_cast<const T*>(p.v) + (int64_t)b * p.sv.b + (int64_t)h * p.sv.h;
     const E* bp = nullptr;
-    if (BIAS != 0) bp = reinterpret_cast<const E*>(p.bias) + (int64_t)b * p.sbias.b + (int64_t)h * p.sbias.h;
+    if (TB != 0) bp = reinterpret_cast<const E*>(p.bias) + (int64_t)b * p.sbias.b + (int64_t)h * p.sbias.h;
+    // ALiBi: the slope of this head and the position of this lane's query row on the key axis
+    float neg_slope = 0.f, ratio = 0.f;
+    if (BIAS == 5) {
+        neg_slope = -reinterpret_cast<const float*>(p.bias)[h];
+        ratio = (float)p.N / (float)p.M;
+    }
 
     // Q^T as B operand: column my_m, k = d
     T8 qreg[C::KSTEPS];
@@ -80,7 +87,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_
         for (int i = 0; i < 16; i++) o_acc[db][i] = 0.f;
 
     const unsigned rows_l = SW::rows_lane(lane), cols_l = SW::cols_lane(lane);
-    KeyStream<T, D, BIAS> ks_;
+    KeyStream<T, D, stream_kind(BIAS)> ks_;
     ks_.init(smem, kp, vp, bp, p.sk.s, p.sv.s, p.sbias.m, p.sbias.n, M, N, mw, wave, lane);
 
     // One step of the K/V stream.  Interior steps (every key in range and visible to every row of
@@ -93,7 +100,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_
         ks_.template begin_step<BV>(k);
         const unsigned k_rows = ks_.k_addr(k) + rows_l, v_cols = ks_.v_addr(k) + cols_l;  // operand reads by address
         const unsigned char* b_lds = ks_.b_lds(k);
-        static_assert(BIAS == 0 || C::NH == 1, "a bias slot covers one 32-key block");
+        static_assert(TB == 0 || C::NH == 1, "a bias slot covers one 32-key block");
         // The step is consumed 32 keys at a time, each block with its own softmax step.  In interior
         // steps of more than one block all score products are issued up front: the MFMAs of the later
         // blocks then run while the vector pipeline works on the first.
@@ -149,6 +156,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_
         auto softmax_step = [&](auto masked_tag) {
             constexpr bool MASKED = decltype(masked_tag)::value;
             float mx = -INFINITY;
+            const float mf = (float)my_m, nf0 = (float)(n0 + nh + 4 * g);  // ALiBi: row and first key as floats
 #pragma unroll
             for (int q4 = 0; q4 < 4; q4++) {
                 const int nl = 8 * q4 + 4 * g;            // first of 4 consecutive keys
@@ -167,6 +175,9 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_
                     f32x4 w = *reinterpret_cast<const f32x4*>(b_lds + ks_.b_off(r, nl));
 #pragma unroll
                     for (int e = 0; e < 4; e++) bv[e] = w[e];
+                } else if constexpr (BIAS == 5) {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) bv[e] = alibi_bias(neg_slope, ratio, mf, nf0 + (float)(8 * q4 + e));
                 }
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
@@ -253,7 +264,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, BIAS>::MIN_BLOCKS)) void fa_fwd_
 #pragma unroll 1
         for (int k = n_fast; k < n_steps; k++) kv_step(k, std::true_type{}, bv_tag);
     };
-    if (BIAS != 0 && p.bias_vec) run(std::true_type{});
+    if (TB != 0 && p.bias_vec) run(std::true_type{});
     else run(std::false_type{});
 
     // ---- epilogue (flash_attention.py:188-194) ----
@@ -297,6 +308,7 @@ template <typename T, int D> static hipError_t launch_bias(const FwdParams& p, i
         FA_CASE(2)
         FA_CASE(3)
         FA_CASE(4)
+        FA_CASE(5)
     }
 #undef FA_CASE
     return hipErrorInvalidValue;

@@ -37,6 +37,7 @@ struct BwdParams {
     const void* bias;
     const float* lse;  // (B, H, M)
     float* delta;      // (B, H, M)        workspace
+    float* partials;   // workspace behind delta: reduced-dBias partial sums (see fa_bwd_kernel)
     void* dq;
     void* dk;
     void* dv;

@@ -23,10 +23,22 @@ import torch
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, GB/s
 MFMA_PEAK_TFLOPS = 2516.6    # MI355X dense bf16/fp16 MFMA, TFLOP/s
-# HBM bytes per launch of the roofline kernel on the headline workload: rocprofv3 FETCH_SIZE and
-# WRITE_SIZE, each scaled by what the same counter reads for a plain 1 GiB copy
-# (profiles/fa_kernels_c3_hbm_traffic.txt: 1.209 GB read + 1.141 GB written)
-ROOFLINE_KERNEL_TRAFFIC_BYTES = 2.350e9
+# HBM bytes per launch of the roofline kernel on the headline workload come from a committed counter
+# summary (rocprofv3 FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter reads for a plain
+# 1 GiB copy); its line "traffic_bytes_per_launch: <number>" is what `roofline.traffic` reports
+TRAFFIC_SUMMARY = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "fa_kernels_c3_hbm_traffic.txt")
+
+
+def measured_traffic_bytes():
+    """The figure of the counter summary, or None when the file or the line is missing."""
+    try:
+        with open(TRAFFIC_SUMMARY) as f:
+            for line in f:
+                if line.startswith("traffic_bytes_per_launch:"):
+                    return float(line.split(":", 1)[1].split()[0])
+    except OSError:
+        pass
+    return None
 
 
 def log(*a):
@@ -81,6 +93,20 @@ def make_config(name, dev):
         bias = (-slopes[:, None, None] * (i * N / M - j).abs())[None].bfloat16().requires_grad_(True)
         return dict(q=rn(B, M, H, D), k=rn(B, N, H, D), v=rn(B, N, H, D), do=rn(B, M, H, D), bias=bias, causal=False,
                     dims=(B, H, M, N, D), bias_es=2, trainable=True)
+    if name == "C5_alibi_in_kernel":
+        # the same attention with the bias formed from indices inside the kernels (no bias tensor,
+        # the gradient is that of the 32 slopes)
+        from triton_flashattn_amd import AlibiBias
+        B, H, M, N, D = 1, 32, 1024, 8192, 128
+        slopes = (2.0 ** (-8.0 * (torch.arange(H, device=dev) + 1) / H)).float().requires_grad_(True)
+        return dict(q=rn(B, M, H, D), k=rn(B, N, H, D), v=rn(B, N, H, D), do=rn(B, M, H, D), bias=AlibiBias(slopes),
+                    causal=False, dims=(B, H, M, N, D), bias_es=0, trainable=True)
+    if name == "C3_row_broadcast_bias":
+        # trainable bias (1, H, 1, N): gradient reduced inside the dK/dV kernel
+        B, M, N, H, D = 2, 4096, 4096, 16, 128
+        return dict(q=rn(B, M, H, D), k=rn(B, N, H, D), v=rn(B, N, H, D), do=rn(B, M, H, D),
+                    bias=rn(1, H, 1, N).requires_grad_(True), causal=False, dims=(B, H, M, N, D), bias_es=0,
+                    trainable=True)
     raise ValueError(name)
 
 
@@ -105,16 +131,24 @@ def time_stages(cfg, iters):
     import triton_flashattn_amd.flash_attention as fa
     from triton_flashattn_amd import _native
     q, k, v, do, bias, causal = cfg["q"], cfg["k"], cfg["v"], cfg["do"], cfg["bias"], cfg["causal"]
-    D = q.shape[-1]
+    B, M, H, D = q.shape
+    N = k.shape[1]
     scale = D ** -0.5
-    b = None if bias is None else bias.detach()
-    t_fwd = event_time_ms(lambda: fa._flash_attn_fwd(q, k, v, b, causal, scale), iters)
-    o, lse = fa._flash_attn_fwd(q, k, v, b, causal, scale)
+    alibi = isinstance(bias, fa.AlibiBias)
+    fwd_bias = bias if alibi or bias is None else bias.detach()
+    t_fwd = event_time_ms(lambda: fa._flash_attn_fwd(q, k, v, fwd_bias, causal, scale), iters)
+    o, lse = fa._flash_attn_fwd(q, k, v, fwd_bias, causal, scale)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-    dbias = torch.empty_like(b) if cfg["trainable"] else None
+    if alibi:
+        b = bias.slopes.detach()
+        dbias = torch.empty_like(b)
+    else:
+        b = None if bias is None else bias.detach().expand(B, H, M, N)
+        dbias = torch.empty_like(bias.detach()).expand(B, H, M, N) if cfg["trainable"] else None
     be = fa._backend
-    ws = be.bwd_workspace(q, k, b, causal, scale)
-    run = lambda stages: be.bwd(do, q, k, v, o, b, causal, scale, lse, dq, dk, dv, dbias, stages=stages, workspace=ws)
+    ws = be.bwd_workspace(q, k, b, causal, scale, alibi)
+    run = lambda stages: be.bwd(do, q, k, v, o, b, causal, scale, lse, dq, dk, dv, dbias, stages=stages, workspace=ws,
+                                alibi=alibi)
     t_bwd = event_time_ms(lambda: run(_native.FA_STAGE_ALL), iters)
     run(_native.FA_STAGE_PREP)
     t_main = event_time_ms(lambda: run(_native.FA_STAGE_MAIN), iters)
@@ -128,7 +162,7 @@ def step(cfg):
     k = cfg["k"].detach().requires_grad_(True)
     v = cfg["v"].detach().requires_grad_(True)
     bias = cfg["bias"]
-    if bias is not None and bias.grad is not None:
+    if isinstance(bias, torch.Tensor) and bias.grad is not None:
         bias.grad = None
     out = flash_attention_fn(q, k, v, bias, cfg["causal"])
     out.backward(cfg["do"])
@@ -184,6 +218,9 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run one plain 1 GiB device-to-device copy and exit (reference point for "
                          "the FETCH_SIZE / WRITE_SIZE counters of a profiler)")
+    ap.add_argument("--profile", metavar="CONFIG", default=None,
+                    help="run only forward + backward of one config (C2, C3, C4, C5, C5_alibi_in_kernel ...) "
+                         "--steps times and exit: the command to put under a profiler")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this build runs on ONE GPU (every (batch, head) pair is independent, so more GPUs "
@@ -204,6 +241,14 @@ def main():
         return
     from triton_flashattn_amd import _native
     _native.load()  # fail loudly before timing anything
+
+    if args.profile:
+        cfg = make_config(args.profile, dev)
+        for _ in range(args.warmup + args.steps):
+            step(cfg)
+        torch.cuda.synchronize()
+        log("ran %d forward + backward steps of %s" % (args.warmup + args.steps, args.profile))
+        return
 
     cfg = make_config("C3", dev)
     B, H, M, N, D = cfg["dims"]
@@ -245,7 +290,8 @@ def main():
         "roofline": {
             "kernel": "fa_bwd_kernel<bf16, D=128, bias=bf16, non-causal, dbias>",
             "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBS, "traffic": ROOFLINE_KERNEL_TRAFFIC_BYTES,
+            "frac": achieved / HBM_PEAK_GBS, "traffic": measured_traffic_bytes(),
+            "traffic_source": "profiles/fa_kernels_c3_hbm_traffic.txt",
             "algorithmic_bytes_per_launch": y_main, "avg_launch_ms": t_main,
             # the kernel's own share of the algorithmic backward FLOPs: 4 of the 5 matrix products
             "mfma_frac_same_kernel": 0.8 * f_bwd / (t_main * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS,
@@ -255,7 +301,7 @@ def main():
 
     if not args.no_other_configs:
         others = {}
-        for name in ("C2", "C4", "C4_expanded_mask", "C5"):
+        for name in ("C2", "C4", "C4_expanded_mask", "C5", "C5_alibi_in_kernel", "C3_row_broadcast_bias"):
             del cfg
             torch.cuda.empty_cache()
             cfg = make_config(name, dev)

@@ -16,8 +16,10 @@
  *   bias, dbias  : (B, H, M, N)     any strides, 0 included (an expanded mask works as is)
  *   lse, delta   : (B, H, M) fp32, dense, in log2 units: lse = log2(sum_j 2^(s_ij))
  * Base pointers of q/k/v/o/do/dq/dk/dv and their B/seq/H strides must be multiples of 16 bytes
- * (FA_ERR_LAYOUT otherwise); bias/dbias have no alignment requirement, but rows with unit N
- * stride and 16-byte aligned row starts take the fast path.
+ * (FA_ERR_LAYOUT otherwise; FA_ERR_HEAD_STRIDE for a D stride other than 1); bias/dbias have no
+ * alignment requirement, but rows with unit N stride and 16-byte aligned row starts take the fast
+ * path.  With FA_MI355_VERBOSE set in the environment the library says on stderr, once per process,
+ * when a bias or dbias misses that path and is read or written element by element.
  */
 #ifndef FA_MI355_H
 #define FA_MI355_H
@@ -55,7 +57,11 @@ enum fa_status {
     FA_ERR_WORKSPACE = -6,   /* workspace NULL or smaller than fa_bwd_workspace_bytes() */
     FA_ERR_UNSUPPORTED = -7, /* combination not built into this library */
     FA_ERR_LAUNCH = -8,      /* the HIP runtime rejected a launch (hipGetLastError) */
-    FA_ERR_TOO_LARGE = -9    /* fa_bwd_noalloc: the problem exceeds FA_NOALLOC_MAX_ROWS */
+    FA_ERR_TOO_LARGE = -9,   /* fa_bwd_noalloc: the problem exceeds FA_NOALLOC_MAX_ROWS */
+    FA_ERR_HEAD_STRIDE = -10 /* the head-dim stride of a q/k/v/o/do/dq/dk/dv tensor is not 1.  The reference's
+                                kernels take any (flash_attention.py:91-94, :117-118); these read rows in 16-byte
+                                chunks, so the caller copies such a tensor to unit stride first (the Python
+                                layer of this package does) */
 };
 
 /* Problem description shared by forward and backward.  Strides are in elements. */

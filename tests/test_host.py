@@ -346,6 +346,10 @@ def test_abi_status_codes_and_workspace():
     a.q = a.k = a.v = a.o = a.lse = base
     for s in (a.q_strides, a.k_strides, a.v_strides, a.o_strides):
         s[0], s[1], s[2], s[3] = 64 * 3 * 100, 64 * 3, 64, 2     # head-dim stride 2
+    assert lib.fa_fwd(ctypes.byref(a), None) == _native.FA_ERR_HEAD_STRIDE
+    assert b"contiguous" in lib.fa_strerror(_native.FA_ERR_HEAD_STRIDE)
+    for s in (a.q_strides, a.k_strides, a.v_strides, a.o_strides):
+        s[0], s[1], s[2], s[3] = 64 * 3 * 100, 64 * 3 + 4, 64, 1  # rows that start off a 16-byte boundary
     assert lib.fa_fwd(ctypes.byref(a), None) == -5            # layout
     b = _native.FaBwdArgs()
     b.p = p

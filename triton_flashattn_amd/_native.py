@@ -51,6 +51,7 @@ EXPORTS = ("fa_abi_version", "fa_strerror", "fa_fwd", "fa_bwd_workspace_bytes", 
 FA_STAGE_PREP, FA_STAGE_MAIN, FA_STAGE_DQ, FA_STAGE_ALL, FA_STAGE_DQ_FROM_DBIAS = 1, 2, 4, 7, 8
 FA_NOALLOC_MAX_ROWS = 1 << 20
 FA_ERR_TOO_LARGE = -9
+FA_ERR_HEAD_STRIDE = -10
 
 _lib = None
 

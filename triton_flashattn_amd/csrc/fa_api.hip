@@ -5,6 +5,7 @@
 #include <atomic>
 #include <cstdio>
 #include <cstdlib>
+#include <initializer_list>
 #include <mutex>
 
 #include "../../include/fa_mi355.h"
@@ -96,15 +97,22 @@ int check_problem(const fa_problem& p) {
 }
 
 // 16-byte rule for a (B, seq, H, D) tensor of 2-byte elements; strides of extent-1 dims are free
-bool qkv_layout_ok(const void* ptr, const int64_t s[4], int nb, int ns, int nh) {
-    if (s[3] != 1) return false;
-    if (reinterpret_cast<uintptr_t>(ptr) % 16 != 0) return false;
-    if (nb > 1 && s[0] % 8 != 0) return false;
-    if (ns > 1 && s[1] % 8 != 0) return false;
-    if (nh > 1 && s[2] % 8 != 0) return false;
+// (FA_OK, FA_ERR_HEAD_STRIDE or FA_ERR_LAYOUT)
+int qkv_layout(const void* ptr, const int64_t s[4], int nb, int ns, int nh) {
+    if (s[3] != 1) return FA_ERR_HEAD_STRIDE;
+    if (reinterpret_cast<uintptr_t>(ptr) % 16 != 0) return FA_ERR_LAYOUT;
+    if (nb > 1 && s[0] % 8 != 0) return FA_ERR_LAYOUT;
+    if (ns > 1 && s[1] % 8 != 0) return FA_ERR_LAYOUT;
+    if (nh > 1 && s[2] % 8 != 0) return FA_ERR_LAYOUT;
     // the kernels form 32-bit byte offsets inside a tile of up to 128 rows
-    if (ns > 1 && (s[1] < 0 || s[1] >= (1 << 23))) return false;
-    return true;
+    if (ns > 1 && (s[1] < 0 || s[1] >= (1 << 23))) return FA_ERR_LAYOUT;
+    return FA_OK;
+}
+// the first complaint among several tensors
+int first_bad(std::initializer_list<int> sts) {
+    for (int s : sts)
+        if (s != FA_OK) return s;
+    return FA_OK;
 }
 
 fa::Strides3 s3(const int64_t s[4]) { return fa::Strides3{s[0], s[1], s[2]}; }
@@ -193,6 +201,8 @@ const char* fa_strerror(int status) {
         case FA_ERR_UNSUPPORTED: return "combination not built into this library";
         case FA_ERR_LAUNCH: return "HIP kernel launch failed";
         case FA_ERR_TOO_LARGE: return "fa_bwd_noalloc: the problem exceeds FA_NOALLOC_MAX_ROWS";
+        case FA_ERR_HEAD_STRIDE:
+            return "the head-dim stride of q, k, v, o, do, dq, dk and dv must be 1: make the tensor contiguous first";
     }
     return "unknown status";
 }
@@ -204,9 +214,9 @@ int fa_fwd(const fa_fwd_args* a, void* stream) {
     if (st != FA_OK) return st;
     if (!a->q || !a->k || !a->v || !a->o || !a->lse) return FA_ERR_NULL;
     if ((p.bias_dtype != FA_BIAS_NONE) != (a->bias != nullptr)) return FA_ERR_NULL;
-    if (!qkv_layout_ok(a->q, a->q_strides, p.B, p.M, p.H) || !qkv_layout_ok(a->k, a->k_strides, p.B, p.N, p.H) ||
-        !qkv_layout_ok(a->v, a->v_strides, p.B, p.N, p.H) || !qkv_layout_ok(a->o, a->o_strides, p.B, p.M, p.H))
-        return FA_ERR_LAYOUT;
+    st = first_bad({qkv_layout(a->q, a->q_strides, p.B, p.M, p.H), qkv_layout(a->k, a->k_strides, p.B, p.N, p.H),
+                    qkv_layout(a->v, a->v_strides, p.B, p.N, p.H), qkv_layout(a->o, a->o_strides, p.B, p.M, p.H)});
+    if (st != FA_OK) return st;
 
     fa::FwdParams k{};
     k.q = a->q; k.k = a->k; k.v = a->v; k.bias = a->bias; k.o = a->o; k.lse = a->lse;
@@ -249,12 +259,13 @@ int bwd_enqueue(const fa_bwd_args* a, void* stream, int stages, float* delta) {
     if (a->dbias && (p.bias_dtype == FA_BIAS_NONE || p.bias_dtype == FA_BIAS_BOOL)) return FA_ERR_DTYPE;
     const int db_mode = dbias_mode(a);
     if (db_mode < 0) return FA_ERR_LAYOUT;
-    if (!qkv_layout_ok(a->q, a->q_strides, p.B, p.M, p.H) || !qkv_layout_ok(a->k, a->k_strides, p.B, p.N, p.H) ||
-        !qkv_layout_ok(a->v, a->v_strides, p.B, p.N, p.H) || !qkv_layout_ok(a->o, a->o_strides, p.B, p.M, p.H) ||
-        !qkv_layout_ok(a->dout, a->do_strides, p.B, p.M, p.H) ||
-        (need_dq && !qkv_layout_ok(a->dq, a->dq_strides, p.B, p.M, p.H)) ||
-        (need_dkv && (!qkv_layout_ok(a->dk, a->dk_strides, p.B, p.N, p.H) || !qkv_layout_ok(a->dv, a->dv_strides, p.B, p.N, p.H))))
-        return FA_ERR_LAYOUT;
+    st = first_bad({qkv_layout(a->q, a->q_strides, p.B, p.M, p.H), qkv_layout(a->k, a->k_strides, p.B, p.N, p.H),
+                    qkv_layout(a->v, a->v_strides, p.B, p.N, p.H), qkv_layout(a->o, a->o_strides, p.B, p.M, p.H),
+                    qkv_layout(a->dout, a->do_strides, p.B, p.M, p.H),
+                    need_dq ? qkv_layout(a->dq, a->dq_strides, p.B, p.M, p.H) : FA_OK,
+                    need_dkv ? qkv_layout(a->dk, a->dk_strides, p.B, p.N, p.H) : FA_OK,
+                    need_dkv ? qkv_layout(a->dv, a->dv_strides, p.B, p.N, p.H) : FA_OK});
+    if (st != FA_OK) return st;
     float* partials = nullptr;
     if (!delta) {
         size_t need = fa_bwd_workspace_bytes(&p);

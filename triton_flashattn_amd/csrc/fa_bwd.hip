@@ -73,7 +73,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, stream_kind(BIAS)>::MIN_BLOCKS))
     const int r = lane & 31, g = lane >> 5;
 
     int mt, bh;
-    decode_block(blockIdx.x, p.n_mtiles, p.B * p.H, mt, bh);
+    decode_block<CAUSAL>(blockIdx.x, p.n_mtiles, p.B * p.H, mt, bh);
     if (CAUSAL) mt = p.n_mtiles - 1 - mt;  // longest rows first
     const int b = bh / p.H, h = bh % p.H;
     const int M = p.M, N = p.N;
@@ -437,7 +437,7 @@ __global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
     const unsigned lds_base = lds_addr_of(smem);
 
     int nt, bh;
-    decode_block(blockIdx.x, p.n_ntiles, p.B * p.H, nt, bh);
+    decode_block<CAUSAL>(blockIdx.x, p.n_ntiles, p.B * p.H, nt, bh);
     const int b = bh / p.H, h = bh % p.H;
     const int M = p.M, N = p.N;
     const int n0 = nt * BN;

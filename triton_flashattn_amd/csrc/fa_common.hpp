@@ -458,11 +458,25 @@ template <typename T, int D, int BIAS, bool WITH_V = true> struct KeyStream {
 // Work-group id -> (tile, batch*head).  Work-groups are dealt round-robin to the 8 XCDs; when
 // the number of (batch, head) pairs is a multiple of 8 every tile of one pair is sent to the same
 // XCD so that its K/V (or Q/dO) stay in that XCD's L2.
+// TILE_MAJOR = false: all tiles of a pair are consecutive (one pair at a time per XCD: the
+// streams of a kernel that reads a bias stay together).  TILE_MAJOR = true: tile t of every pair
+// comes before tile t + 1 of any; the causal kernels, whose tiles are numbered longest first,
+// so start all long tiles before any short one (a greedy schedule with the longest jobs first
+// ends near the average load, one that mixes them ends up to one long tile later).
+template <bool TILE_MAJOR = false>
 __device__ __forceinline__ void decode_block(int id, int n_tiles, int BH, int& tile, int& bh) {
     if ((BH & 7) == 0) {
-        int xcd = id & 7, slot = id >> 3;
-        bh = (slot / n_tiles) * 8 + xcd;
-        tile = slot % n_tiles;
+        const int xcd = id & 7, slot = id >> 3, per_xcd = BH >> 3;
+        if (TILE_MAJOR) {
+            tile = slot / per_xcd;
+            bh = (slot % per_xcd) * 8 + xcd;
+        } else {
+            bh = (slot / n_tiles) * 8 + xcd;
+            tile = slot % n_tiles;
+        }
+    } else if (TILE_MAJOR) {
+        tile = id / BH;
+        bh = id % BH;
     } else {
         bh = id / n_tiles;
         tile = id % n_tiles;

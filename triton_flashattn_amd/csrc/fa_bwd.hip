@@ -356,9 +356,19 @@ template <> struct BiasQuad<4> {
 };
 
 // ---------------------------------------------------------------------------------------------
-template <int D, int BIAS> struct BwdCfg {
+// OCC2: two work-groups per CU (four waves per SIMD, 128 registers each, half of the LDS): the
+// configuration of the small head dims without a float bias, whose blocks are small enough.
+constexpr bool bwd_occ2(int D, int bias) {
+#ifdef FA_EXP_NO_OCC2
+    return false;
+#else
+    return D <= 64 && bias == 0;
+#endif
+}
+template <int D, int BIAS, bool OCC2 = false> struct BwdCfg {
     static constexpr int BN = 128, NT = 512;
-    static constexpr int NSUB = (D <= 64 && BIAS == 0) ? 2 : 1;  // 32-row sub-blocks of a query block
+    static constexpr int LDS_LIMIT = OCC2 ? 81920 : 163840;
+    static constexpr int NSUB = (D <= 64 && BIAS == 0 && !OCC2) ? 2 : 1;  // 32-row sub-blocks of a query block
     static constexpr int BMI = 32 * NSUB;
     static constexpr int DP = D < 32 ? 32 : D;
     static constexpr int DB = DP / 32;
@@ -385,8 +395,8 @@ template <int D, int BIAS> struct BwdCfg {
     static constexpr int lds_total(int la, int defer) {
         return (2 * la + 3 + defer) * (Q_BYTES + BMI * 4) + DS_BYTES + 2 * P_BYTES + 4 * (la + 1) * BT_BYTES;
     }
-    static constexpr int LA = D > 128 ? 1 : (lds_total(3, 1) <= 163840 ? 3 : 2);
-    static constexpr bool DEFER_DK = D <= 128 && lds_total(LA, 1) <= 163840;
+    static constexpr int LA = D > 128 ? 1 : (lds_total(3, 1) <= LDS_LIMIT ? 3 : 2);
+    static constexpr bool DEFER_DK = D <= 128 && lds_total(LA, 1) <= LDS_LIMIT;
     static constexpr int NDOB = LA + 1;                    // dO (+delta) buffers
     static constexpr int RING = LA + 1;                    // bias slots per S-wave
     static constexpr int NQB = LA + 2 + (DEFER_DK ? 1 : 0);  // Q (+LSE) buffers
@@ -398,6 +408,8 @@ template <int D, int BIAS> struct BwdCfg {
     static constexpr int OFF_BIAS = OFF_DELTA + NDOB * BMI * 4;
     static constexpr int LOOP_BYTES = OFF_BIAS + 4 * RING * BT_BYTES;
     static constexpr int LDS_BYTES = LOOP_BYTES;
+    static_assert(LDS_BYTES <= LDS_LIMIT, "LDS budget of the configuration");
+    static constexpr int WAVES_PER_SIMD = OCC2 ? 4 : 2;
 };
 
 // Work split inside a work-group of 8 waves.  Waves 0-3 ("S-waves") and waves 4-7 ("dP-waves")
@@ -416,9 +428,9 @@ template <int D, int BIAS> struct BwdCfg {
 // query rows, one fp32 per (batch, head, key), for ALiBi the gradient of the slope, one fp32 per
 // (batch, head, key tile, wave); a second small kernel sums those over the broadcast dimensions.
 template <typename T, int D, int BIAS, bool CAUSAL, int DBIAS>
-__global__ __launch_bounds__(512, 2) void fa_bwd_kernel(const BwdParams p) {
+__global__ __launch_bounds__(512, (BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>::WAVES_PER_SIMD)) void fa_bwd_kernel(const BwdParams p) {
     constexpr int TB = tile_kind(BIAS);  // kind of bias tile that is streamed (none for ALiBi)
-    typedef BwdCfg<D, TB> C;
+    typedef BwdCfg<D, TB, bwd_occ2(D, BIAS)> C;
     typedef Swz<D> SW;
     typedef typename VecOf<T>::v8 T8;
     typedef typename VecOf<T>::v4 T4;

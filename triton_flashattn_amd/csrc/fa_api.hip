@@ -288,6 +288,9 @@ int bwd_enqueue(const fa_bwd_args* a, void* stream, int stages, float* delta) {
         k.sbias = s4(a->bias_strides);
         k.bias_vec = bias_vec_ok(a->bias, a->bias_strides, p) ? 1 : 0;
     }
+    // a bias that does not depend on the query row: the dK/dV kernel keeps it in one register per key
+    if (a->bias && p.bias_dtype >= FA_BIAS_BOOL && p.bias_dtype <= FA_BIAS_F32 && (p.M == 1 || a->bias_strides[2] == 0))
+        k.row_bias_kind = p.bias_dtype;
     if (a->dbias && p.bias_dtype != FA_BIAS_ALIBI) {
         k.sdbias = s4(a->dbias_strides);
         k.dbias_vec = db_mode == 1 && bias_vec_ok(a->dbias, a->dbias_strides, p) ? 1 : 0;

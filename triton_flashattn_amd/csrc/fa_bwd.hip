@@ -346,6 +346,8 @@ template <> struct BiasQuad<5> {  // ALiBi: nothing to read, the kernel computes
     __device__ __forceinline__ void load(const unsigned char*, int, int, int) {}
     __device__ __forceinline__ float get(int) const { return 0.f; }
 };
+template <> struct BiasQuad<6> : BiasQuad<5> {};  // row-broadcast bias: one value per key, held by the kernel
+template <> struct BiasQuad<7> : BiasQuad<5> {};
 template <> struct BiasQuad<4> {
     float v[4];
     __device__ __forceinline__ void load(const unsigned char* slice, int row0, int key, int) {
@@ -362,7 +364,7 @@ constexpr bool bwd_occ2(int D, int bias) {
 #ifdef FA_EXP_NO_OCC2
     return false;
 #else
-    return D <= 64 && bias == 0;
+    return D <= 64 && (bias == 0 || bias == 6 || bias == 7);
 #endif
 }
 template <int D, int BIAS, bool OCC2 = false> struct BwdCfg {
@@ -471,6 +473,20 @@ __global__ __launch_bounds__(512, (BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>
         neg_slope = -reinterpret_cast<const float*>(p.bias)[h];
         ratio = (float)p.N / (float)p.M;
     }
+    // row-broadcast bias: the term of this lane's key, natural units (6) or 0 / mask value in log2 units (7)
+    float row_bv = 0.f;
+    if (BIAS == 6 || BIAS == 7) {
+        if (my_n < N) {
+            const int64_t idx = (int64_t)b * p.sbias.b + (int64_t)h * p.sbias.h + (int64_t)my_n * p.sbias.n;
+            switch (p.row_bias_kind) {
+                case 1: row_bv = reinterpret_cast<const unsigned char*>(p.bias)[idx] ? 0.f : kMask; break;
+                case 2: row_bv = (float)reinterpret_cast<const _Float16*>(p.bias)[idx]; break;
+                case 3: row_bv = (float)reinterpret_cast<const __bf16*>(p.bias)[idx]; break;
+                default: row_bv = reinterpret_cast<const float*>(p.bias)[idx]; break;
+            }
+        }
+    }
+    constexpr bool NATURAL = BIAS >= 2 && BIAS != 7;  // the bias term is in natural units (else log2 units)
     unsigned char* ring_lds = smem + C::OFF_BIAS + kb * C::RING * C::BT_BYTES;
     float* p_lds = reinterpret_cast<float*>(smem + C::OFF_P) + kb * NSUB * 64 * 16;  // + buffer * P_BYTES / 4
 
@@ -748,6 +764,7 @@ __global__ __launch_bounds__(512, (BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>
                                 // bool mask: the additive term in log2 units; float bias: natural units
                                 float bv = bias_in[sb][q4].get(e);
                                 if constexpr (BIAS == 5) bv = alibi_bias(neg_slope, ratio, mf0 + (float)(ml0 - 4 * g + e), (float)my_n);
+                                if constexpr (BIAS == 6 || BIAS == 7) bv = row_bv;
                                 float pv;
                                 if constexpr (MASKED) {
                                     const int m = m0 + ml0 + e;
@@ -755,12 +772,12 @@ __global__ __launch_bounds__(512, (BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>
                                     const bool oob = (m >= M) || (my_n >= N);
                                     float tmask = oob ? kMask : 0.f;
                                     if (CAUSAL) tmask += (m < my_n) ? kMask : 0.f;
-                                    float add = BIAS >= 2 ? __fmul_rn(bv, kLog2e) : bv;
+                                    float add = NATURAL ? __fmul_rn(bv, kLog2e) : bv;
                                     if (BIAS != 0) add = oob ? kMask : add;  // out-of-range bias reads as masked
                                     x = __fadd_rn(x, __fadd_rn(tmask, add));
                                     pv = fast_exp2(x - lse4[e]);
                                 } else {
-                                    const float off = BIAS >= 2 ? __builtin_fmaf(bv, kLog2e, -lse4[e]) : bv - lse4[e];
+                                    const float off = NATURAL ? __builtin_fmaf(bv, kLog2e, -lse4[e]) : bv - lse4[e];
                                     pv = fast_exp2(__builtin_fmaf(sacc[sb][i], qk_scale, off));
                                 }
                                 p4[e] = pv;
@@ -1059,9 +1076,14 @@ template <typename T, int D> static hipError_t launch_all(const BwdParams& p, in
     }
     if (stages & 2) {
 #define FA_CASE(BK, DBK)                                                                                      \
-    if (bias == BK && dbias == DBK)                                                                           \
+    if (kbias == BK && dbias == DBK)                                                                          \
         e = causal ? launch_main<T, D, BK, true, DBK>(p, st) : launch_main<T, D, BK, false, DBK>(p, st);
+    // a bias that is the same for every query row is one register per key for this kernel
+    const int kbias = (p.row_bias_kind != 0 && dbias != 1) ? (p.row_bias_kind == 1 ? 7 : 6) : bias;
     FA_CASE(0, 0)
+    else FA_CASE(6, 0)
+    else FA_CASE(6, 2)
+    else FA_CASE(7, 0)
     else FA_CASE(1, 0)
     else FA_CASE(2, 0)
     else FA_CASE(2, 1)

@@ -251,11 +251,15 @@ template <> struct BiasElem<3> { typedef __bf16 type; };
 template <> struct BiasElem<4> { typedef float type; };
 template <> struct BiasElem<5> { typedef float type; };  // ALiBi: one fp32 slope per head, no tile
 template <> struct BiasElem<6> { typedef unsigned char type; };  // the stream kind of ALiBi (below)
+template <> struct BiasElem<7> { typedef unsigned char type; };
 
 // Bias kind 5 (ALiBi): bias[b,h,i,j] = -slope[h] * |i * N / M - j| is computed from the indices, so no
 // bias tile exists and the K/V stream is tiled as without a bias.  TILE_KIND maps a bias kind to
 // the kind of tile that StreamCfg / KeyStream handle.
-constexpr int tile_kind(int bias) { return bias == 5 ? 0 : bias; }
+// Kinds 6 and 7 exist in the dK/dV kernel only: a float bias / a bool mask that is the same for every
+// query row (stride 0 along M).  There the lane is the key, so the whole bias of a wave is ONE
+// register per lane, read once, and nothing is streamed.
+constexpr int tile_kind(int bias) { return bias >= 5 ? 0 : bias; }
 // ... and to the kind that StreamCfg / KeyStream tile the K/V stream for: 6 = no bias tile, but steps of
 // 32 keys like the kernels with one (the element-wise work of ALiBi needs the registers that the
 // 64-key steps of the bias-free kernels spend on a second block of scores)

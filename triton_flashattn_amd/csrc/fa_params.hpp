@@ -50,6 +50,8 @@ struct BwdParams {
     int n_mtiles;   // query tiles of the dQ kernel
     int bias_vec;   // bias rows may be read with aligned 16-byte loads
     int dbias_vec;  // dbias rows may be written with aligned 16-byte stores
+    int row_bias_kind;  // 0, or the element kind (1 bool, 2 fp16, 3 bf16, 4 fp32) of a bias with stride 0 along M
+                        // that the dK/dV kernel reads as one value per key
 };
 
 }  // namespace fa

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define FA_ABI_VERSION 2
+#define FA_ABI_VERSION 3
 
 /* element type of q, k, v, o and their gradients */
 enum fa_dtype { FA_F16 = 0, FA_BF16 = 1 };
@@ -81,6 +81,8 @@ typedef struct fa_fwd_args {
     float *lse;                   /* (B, H, M) */
     int64_t q_strides[4], k_strides[4], v_strides[4], o_strides[4]; /* (B, seq, H, D) */
     int64_t bias_strides[4];      /* (B, H, M, N) */
+    void *workspace;              /* optional (may be NULL): fa_fwd_workspace_bytes() bytes, 256-byte aligned */
+    size_t workspace_bytes;
 } fa_fwd_args;
 
 /* _flash_attn_bwd: flash_attention.py:688-763.  dq, dk, dv (and dbias when non-NULL, i.e. when
@@ -120,6 +122,13 @@ int fa_fwd(const fa_fwd_args *args, void *stream);
 /* Bytes of scratch the backward needs for this problem: delta, (B, H, M) fp32
  * (flash_attention.py:689), followed by the partial sums of the reduced dbias layouts. */
 size_t fa_bwd_workspace_bytes(const fa_problem *p);
+
+/* Scratch with which fa_fwd splits the keys of a query tile between several work-groups and merges
+ * their softmaxes (the outputs of the shares in the element type of q, and their LSEs); 0 when the
+ * problem has enough query tiles to fill the GPU, or is causal.  No counterpart in the reference (its grid is one program
+ * per query tile, flash_attention.py:668).  The workspace is optional: without it fa_fwd runs one
+ * work-group per query tile, with the same results up to fp32 rounding of the merge. */
+size_t fa_fwd_workspace_bytes(const fa_problem *p);
 
 /* Enqueue the backward (delta, dK/dV/dBias/dQ) on `stream`.
  * Replaces _flash_attn_bwd, flash_attention.py:688-763 (K and bias pre-scale :699-704 included). */

@@ -316,19 +316,26 @@ def test_library_exports_every_declared_symbol():
 def test_struct_layouts_match_header():
     # sizes follow from the C declaration: 9 x 4 bytes; pointers + strides
     assert ctypes.sizeof(_native.FaProblem) == 36
-    assert ctypes.sizeof(_native.FaFwdArgs) == 40 + 6 * 8 + 5 * 32
+    assert ctypes.sizeof(_native.FaFwdArgs) == 40 + 6 * 8 + 5 * 32 + 16
     assert ctypes.sizeof(_native.FaBwdArgs) == 40 + 12 * 8 + 8 + 10 * 32
 
 
 def test_abi_status_codes_and_workspace():
     lib = _native.load()
-    assert lib.fa_abi_version() == 2
+    assert lib.fa_abi_version() == 3
     assert lib.fa_strerror(0) == b"ok"
     assert b"head dimension" in lib.fa_strerror(-3)
     p = _native.FaProblem(B=2, H=3, M=100, N=50, D=64, dtype=_native.FA_BF16, bias_dtype=0, causal=0, sm_scale=0.1)
     rows = 2 * 3 * 100
     pad = lambda x: (x + 255) // 256 * 256
     assert lib.fa_bwd_workspace_bytes(ctypes.byref(p)) == pad(rows * 4) + pad(2 * 3 * 50 * 4)   # delta + partial sums
+    assert lib.fa_fwd_workspace_bytes(ctypes.byref(p)) == 0            # too few keys to split
+    few = _native.FaProblem(B=1, H=32, M=1024, N=8192, D=128, dtype=_native.FA_BF16, bias_dtype=3, causal=0, sm_scale=0.1)
+    assert lib.fa_fwd_workspace_bytes(ctypes.byref(few)) == pad(2 * 32 * 1024 * 128 * 2) + pad(2 * 32 * 1024 * 4)  # two shares
+    few.causal, few.N = 1, 1024
+    assert lib.fa_fwd_workspace_bytes(ctypes.byref(few)) == 0            # never when causal
+    many = _native.FaProblem(B=2, H=16, M=4096, N=4096, D=128, dtype=_native.FA_BF16, bias_dtype=3, causal=0, sm_scale=0.1)
+    assert lib.fa_fwd_workspace_bytes(ctypes.byref(many)) == 0           # enough query tiles
     a = _native.FaFwdArgs()
     a.p = p
     assert lib.fa_fwd(ctypes.byref(a), None) == -1            # NULL pointers

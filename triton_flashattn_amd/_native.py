@@ -7,7 +7,7 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libfa_mi355.so")
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 FA_F16, FA_BF16 = 0, 1
 FA_BIAS_NONE, FA_BIAS_BOOL, FA_BIAS_F16, FA_BIAS_BF16, FA_BIAS_F32, FA_BIAS_ALIBI = 0, 1, 2, 3, 4, 5
@@ -30,6 +30,7 @@ class FaFwdArgs(ctypes.Structure):
         ("o", ctypes.c_void_p), ("lse", ctypes.c_void_p),
         ("q_strides", _i64x4), ("k_strides", _i64x4), ("v_strides", _i64x4), ("o_strides", _i64x4),
         ("bias_strides", _i64x4),
+        ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
     ]
 
 
@@ -46,10 +47,11 @@ class FaBwdArgs(ctypes.Structure):
     ]
 
 
-EXPORTS = ("fa_abi_version", "fa_strerror", "fa_fwd", "fa_bwd_workspace_bytes", "fa_bwd", "fa_bwd_stages",
+EXPORTS = ("fa_abi_version", "fa_strerror", "fa_fwd", "fa_fwd_workspace_bytes", "fa_bwd_workspace_bytes", "fa_bwd", "fa_bwd_stages",
            "fa_bwd_noalloc")
 FA_STAGE_PREP, FA_STAGE_MAIN, FA_STAGE_DQ, FA_STAGE_ALL, FA_STAGE_DQ_FROM_DBIAS = 1, 2, 4, 7, 8
 FA_NOALLOC_MAX_ROWS = 1 << 20
+FA_ERR_WORKSPACE = -6
 FA_ERR_TOO_LARGE = -9
 FA_ERR_HEAD_STRIDE = -10
 
@@ -76,6 +78,8 @@ def load():
     lib.fa_strerror.argtypes = [ctypes.c_int]
     lib.fa_fwd.restype = ctypes.c_int
     lib.fa_fwd.argtypes = [ctypes.POINTER(FaFwdArgs), ctypes.c_void_p]
+    lib.fa_fwd_workspace_bytes.restype = ctypes.c_size_t
+    lib.fa_fwd_workspace_bytes.argtypes = [ctypes.POINTER(FaProblem)]
     lib.fa_bwd_workspace_bytes.restype = ctypes.c_size_t
     lib.fa_bwd_workspace_bytes.argtypes = [ctypes.POINTER(FaProblem)]
     lib.fa_bwd.restype = ctypes.c_int

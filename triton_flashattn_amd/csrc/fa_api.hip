@@ -167,6 +167,25 @@ size_t partial_floats(const fa_problem& p) {
     return (size_t)p.B * p.H * ((size_t)p.N > tiles4 ? (size_t)p.N : tiles4);
 }
 
+// Keys of a query tile split between work-groups when the query tiles alone leave the GPU half empty
+// (fewer than two work-groups per CU): as many splits as it takes to get there, at most four, each
+// with at least 16 steps of the K/V stream.
+struct FwdSplit {
+    int n_splits, keys_per_split;
+};
+FwdSplit fwd_split(const fa_problem& p) {
+    if (p.causal) return {1, 0};
+    const int64_t wgs = (int64_t)((p.M + fa::fwd_block_m() - 1) / fa::fwd_block_m()) * p.B * p.H;
+    if (wgs >= 512) return {1, 0};
+    const int bk = p.bias_dtype == FA_BIAS_NONE ? 64 : 32;  // keys per step of the forward kernel
+    const int n_steps = (p.N + bk - 1) / bk;
+    int s = (int)(512 / wgs);
+    s = s > 4 ? 4 : s;
+    while (s > 1 && n_steps / s < 16) s--;
+    if (s <= 1) return {1, 0};
+    return {s, (n_steps + s - 1) / s * bk};
+}
+
 // How dbias is laid out: 0 none, 1 dense (B, H, M, N), 2 reduced in the kernels; -1 = not acceptable
 int dbias_mode(const fa_bwd_args* a) {
     const fa_problem& p = a->p;
@@ -207,6 +226,14 @@ const char* fa_strerror(int status) {
     return "unknown status";
 }
 
+size_t fa_fwd_workspace_bytes(const fa_problem* p) {
+    if (!p || check_problem(*p) != FA_OK) return 0;
+    const FwdSplit s = fwd_split(*p);
+    if (s.n_splits <= 1) return 0;
+    const size_t rows = (size_t)p->B * p->H * p->M;
+    return align256((size_t)s.n_splits * rows * p->D * 2) + align256((size_t)s.n_splits * rows * sizeof(float));
+}
+
 int fa_fwd(const fa_fwd_args* a, void* stream) {
     if (!a) return FA_ERR_NULL;
     const fa_problem& p = a->p;
@@ -229,6 +256,19 @@ int fa_fwd(const fa_fwd_args* a, void* stream) {
         if (!k.bias_vec) note_slow_bias("bias", a->bias, a->bias_strides, p);
     }
     k.n_mtiles = (p.M + fa::fwd_block_m() - 1) / fa::fwd_block_m();
+    k.n_splits = 1;
+    if (a->workspace) {
+        const size_t need = fa_fwd_workspace_bytes(&p);
+        if (need > 0) {
+            if (a->workspace_bytes < need || reinterpret_cast<uintptr_t>(a->workspace) % 256 != 0) return FA_ERR_WORKSPACE;
+            const FwdSplit s = fwd_split(p);
+            const size_t rows = (size_t)p.B * p.H * p.M;
+            k.n_splits = s.n_splits;
+            k.keys_per_split = s.keys_per_split;
+            k.part_o = a->workspace;
+            k.part_lse = reinterpret_cast<float*>(static_cast<char*>(a->workspace) + align256((size_t)s.n_splits * rows * p.D * 2));
+        }
+    }
     hipError_t e = fa::launch_fwd(k, p.D, p.dtype, p.bias_dtype, p.causal != 0, static_cast<hipStream_t>(stream));
     if (e == hipErrorNotSupported) return FA_ERR_UNSUPPORTED;
     return e == hipSuccess ? FA_OK : FA_ERR_LAUNCH;

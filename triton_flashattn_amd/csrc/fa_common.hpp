@@ -407,16 +407,17 @@ template <typename T, int D, int BIAS, bool WITH_V = true> struct KeyStream {
     }
     // Before the first step, in the order the steps assume: the first bias slices, then K/V of a
     // step followed by the bias slice issued in the same step.  BV: the bias slices come by copy.
-    template <bool BV> __device__ __forceinline__ void prologue() {
+    // k0: the first step of the stream (0 unless the keys are split between work-groups)
+    template <bool BV> __device__ __forceinline__ void prologue(int k0 = 0) {
         const unsigned saved_m0 = lds_copy_begin();
         if constexpr (BV) {
 #pragma unroll
-            for (int i = 0; i < C::NBS - 1 - C::LA; i++) issue_bias(i);
+            for (int i = 0; i < C::NBS - 1 - C::LA; i++) issue_bias(k0 + i);
         }
 #pragma unroll
         for (int i = 0; i < C::LA; i++) {
-            issue_kv(i);
-            if constexpr (BV) issue_bias(C::NBS - 1 - C::LA + i);
+            issue_kv(k0 + i);
+            if constexpr (BV) issue_bias(k0 + C::NBS - 1 - C::LA + i);
         }
         lds_copy_end(saved_m0);
     }

@@ -43,19 +43,25 @@ __global__ __launch_bounds__(256, (StreamCfg<D, stream_kind(BIAS)>::MIN_BLOCKS))
     const int r = lane & 31, g = lane >> 5;
 
     int mt, bh;
-    decode_block<CAUSAL>(blockIdx.x, p.n_mtiles, p.B * p.H, mt, bh);
+    decode_block<CAUSAL>(blockIdx.x, p.n_mtiles * p.n_splits, p.B * p.H, mt, bh);
+    // With the keys split between work-groups (never when causal) this one sees keys key0 ..
+    // key0 + N - 1 as if they were all there are; only ALiBi needs to know better.
+    const int split = mt % p.n_splits;
+    mt /= p.n_splits;
+    const int key0 = split * p.keys_per_split;
     if (CAUSAL) mt = p.n_mtiles - 1 - mt;  // longest rows first
     const int b = bh / p.H, h = bh % p.H;
-    const int M = p.M, N = p.N;
+    const int M = p.M;
+    const int N = p.n_splits > 1 ? (p.N - key0 < p.keys_per_split ? p.N - key0 : p.keys_per_split) : p.N;
     const int m0 = mt * BM;
     const int mw = m0 + wave * 32;  // first query row of this wave
     const int my_m = mw + r;
 
     const T* qp = reinterpret_cast<const T*>(p.q) + (int64_t)b * p.sq.b + (int64_t)h * p.sq.h;
-    const T* kp = reinterpret_cast<const T*>(p.k) + (int64_t)b * p.sk.b + (int64_t)h * p.sk.h;
-    const T* vp = reinterpret_cast<const T*>(p.v) + (int64_t)b * p.sv.b + (int64_t)h * p.sv.h;
+    const T* kp = reinterpret_cast<const T*>(p.k) + (int64_t)b * p.sk.b + (int64_t)h * p.sk.h + (int64_t)key0 * p.sk.s;
+    const T* vp = reinterpret_cast<const T*>(p.v) + (int64_t)b * p.sv.b + (int64_t)h * p.sv.h + (int64_t)key0 * p.sv.s;
     const E* bp = nullptr;
-    if (TB != 0) bp = reinterpret_cast<const E*>(p.bias) + (int64_t)b * p.sbias.b + (int64_t)h * p.sbias.h;
+    if (TB != 0) bp = reinterpret_cast<const E*>(p.bias) + (int64_t)b * p.sbias.b + (int64_t)h * p.sbias.h + (int64_t)key0 * p.sbias.n;
     // ALiBi: the slope of this head and the position of this lane's query row on the key axis
     float neg_slope = 0.f, ratio = 0.f;
     if (BIAS == 5) {
@@ -156,7 +162,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, stream_kind(BIAS)>::MIN_BLOCKS))
         auto softmax_step = [&](auto masked_tag) {
             constexpr bool MASKED = decltype(masked_tag)::value;
             float mx = -INFINITY;
-            const float mf = (float)my_m, nf0 = (float)(n0 + nh + 4 * g);  // ALiBi: row and first key as floats
+            const float mf = (float)my_m, nf0 = (float)(key0 + n0 + nh + 4 * g);  // ALiBi: row and first key as floats
 #pragma unroll
             for (int q4 = 0; q4 < 4; q4++) {
                 const int nl = 8 * q4 + 4 * g;            // first of 4 consecutive keys
@@ -270,7 +276,10 @@ __global__ __launch_bounds__(256, (StreamCfg<D, stream_kind(BIAS)>::MIN_BLOCKS))
     // ---- epilogue (flash_attention.py:188-194) ----
     const float l_tot = pair_sum(l_i);
     const float inv_l = 1.f / l_tot;
-    if (g == 0 && my_m < M) p.lse[((int64_t)b * p.H + h) * M + my_m] = m_i + fast_log2(l_tot);
+    // one of several shares of the keys: output and LSE go to this share's slice of the scratch
+    const bool shared = p.n_splits > 1;
+    float* lse_out = shared ? p.part_lse + ((int64_t)split * p.B * p.H + bh) * M : p.lse + ((int64_t)b * p.H + h) * M;
+    if (g == 0 && my_m < M) lse_out[my_m] = m_i + fast_log2(l_tot);
 
     ks_.drain();  // K/V slots are dead and no copy is in flight: reuse their LDS for the output tile
     T* o_lds = reinterpret_cast<T*>(smem) + wave * 32 * OS;
@@ -285,16 +294,54 @@ __global__ __launch_bounds__(256, (StreamCfg<D, stream_kind(BIAS)>::MIN_BLOCKS))
         }
     }
     __syncthreads();
-    T* op = reinterpret_cast<T*>(p.o) + (int64_t)b * p.so.b + (int64_t)h * p.so.h;
+    T* op = shared ? reinterpret_cast<T*>(p.part_o) + ((int64_t)split * p.B * p.H + bh) * M * D
+                   : reinterpret_cast<T*>(p.o) + (int64_t)b * p.so.b + (int64_t)h * p.so.h;
+    const int64_t o_stride = shared ? D : p.so.s;
     for (int c = lane; c < 32 * CPR; c += 64) {
         int row = c / CPR, ch = c % CPR;
-        if (mw + row < M) gst16(op + (int64_t)(mw + row) * p.so.s + ch * 8, lds_read16(o_lds + row * OS + ch * 8));
+        if (mw + row < M) gst16(op + (int64_t)(mw + row) * o_stride + ch * 8, lds_read16(o_lds + row * OS + ch * 8));
     }
 }
 
+// out = sum over the shares of 2^(lse_s - lse) out_s with lse = log2 sum 2^lse_s: the softmax over
+// all keys from the softmaxes over the shares.  One thread per 8 head-dim elements of a row.
+template <typename T, int D> __global__ __launch_bounds__(256) void fa_fwd_merge_kernel(const FwdParams p) {
+    typedef typename VecOf<T>::v8 T8;
+    constexpr int TPR = D / 8;
+    const int64_t rows = (int64_t)p.B * p.H * p.M;
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t row = idx / TPR;
+    const int c = (int)(idx % TPR);
+    if (row >= rows) return;
+    float mx = -INFINITY;
+    for (int s = 0; s < p.n_splits; s++) mx = fmaxf(mx, p.part_lse[s * rows + row]);
+    float sum = 0.f;
+    for (int s = 0; s < p.n_splits; s++) sum += fast_exp2(p.part_lse[s * rows + row] - mx);
+    const float lse = mx + fast_log2(sum);
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < p.n_splits; s++) {
+        const float w = fast_exp2(p.part_lse[s * rows + row] - lse);
+        const T8 v = as_vec<T8>(gld16(reinterpret_cast<const T*>(p.part_o) + (s * rows + row) * D + c * 8));
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc[e] += w * (float)v[e];
+    }
+    const int m = (int)(row % p.M);
+    const int64_t bh = row / p.M;
+    const int b = (int)(bh / p.H), h = (int)(bh % p.H);
+    T8 o8;
+#pragma unroll
+    for (int e = 0; e < 8; e++) o8[e] = (T)acc[e];
+    gst16(reinterpret_cast<T*>(p.o) + (int64_t)b * p.so.b + (int64_t)h * p.so.h + (int64_t)m * p.so.s + c * 8, as_raw(o8));
+    if (c == 0) p.lse[row] = lse;
+}
+
 template <typename T, int D, int BIAS, bool CAUSAL> static hipError_t launch_one(const FwdParams& p, hipStream_t st) {
-    dim3 grid((unsigned)(p.n_mtiles * p.B * p.H));
+    dim3 grid((unsigned)(p.n_mtiles * p.n_splits * p.B * p.H));
     hipLaunchKernelGGL((fa_fwd_kernel<T, D, BIAS, CAUSAL>), grid, dim3(256), 0, st, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess || p.n_splits == 1) return e;
+    const int64_t threads = (int64_t)p.B * p.H * p.M * (D / 8);
+    hipLaunchKernelGGL((fa_fwd_merge_kernel<T, D>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, p);
     return hipGetLastError();
 }
 

@@ -26,6 +26,13 @@ struct FwdParams {
     float sm_scale;
     int bias_vec;  // bias rows may be read with aligned 16-byte loads
     int n_mtiles;
+    // Keys split between n_splits work-groups per query tile (1 = no split): split s takes
+    // keys_per_split keys (a multiple of the kernel's step) and writes its output, in the element
+    // type of q, and its LSE to part_o (n_splits, B*H, M, D) / part_lse (n_splits, B*H, M);
+    // fa_fwd_merge_kernel combines them.
+    int n_splits, keys_per_split;
+    void* part_o;
+    float* part_lse;
 };
 
 struct BwdParams {

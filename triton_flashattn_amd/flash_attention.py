@@ -119,6 +119,12 @@ class _HipBackend:
             a.bias = bias.data_ptr()
             if not alibi:
                 a.bias_strides = _strides4(bias)
+        # problems with too few query tiles to fill the GPU split their keys between work-groups and
+        # need scratch for the partial results (only touched by work enqueued on this stream)
+        nbytes = int(lib.fa_fwd_workspace_bytes(ctypes.byref(a.p)))
+        if nbytes > 0:
+            workspace = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+            a.workspace, a.workspace_bytes = workspace.data_ptr(), nbytes
         with torch.cuda.device(dev):
             stream = torch.cuda.current_stream(dev).cuda_stream
             _native.check(lib.fa_fwd(ctypes.byref(a), ctypes.c_void_p(stream)))

@@ -186,6 +186,12 @@ FwdSplit fwd_split(const fa_problem& p) {
     return {s, (n_steps + s - 1) / s * bk};
 }
 
+// the shares of dq of a dQ kernel that splits its keys like the forward (0 when it does not)
+size_t dq_share_bytes(const fa_problem& p) {
+    const FwdSplit s = fwd_split(p);
+    return s.n_splits <= 1 ? 0 : align256((size_t)s.n_splits * p.B * p.H * p.M * p.D * 2);
+}
+
 // How dbias is laid out: 0 none, 1 dense (B, H, M, N), 2 reduced in the kernels; -1 = not acceptable
 int dbias_mode(const fa_bwd_args* a) {
     const fa_problem& p = a->p;
@@ -276,7 +282,7 @@ int fa_fwd(const fa_fwd_args* a, void* stream) {
 
 size_t fa_bwd_workspace_bytes(const fa_problem* p) {
     if (!p || check_problem(*p) != FA_OK) return 0;
-    return align256(delta_floats(*p) * sizeof(float)) + align256(partial_floats(*p) * sizeof(float));
+    return align256(delta_floats(*p) * sizeof(float)) + align256(partial_floats(*p) * sizeof(float)) + dq_share_bytes(*p);
 }
 
 }  // extern "C"
@@ -307,12 +313,20 @@ int bwd_enqueue(const fa_bwd_args* a, void* stream, int stages, float* delta) {
                     need_dkv ? qkv_layout(a->dv, a->dv_strides, p.B, p.N, p.H) : FA_OK});
     if (st != FA_OK) return st;
     float* partials = nullptr;
+    int dq_splits = 1, dq_keys = 0;  // (the entry point without allocations does not split: its scratch is small)
+    void* part_dq = nullptr;
     if (!delta) {
         size_t need = fa_bwd_workspace_bytes(&p);
         if (!a->workspace || a->workspace_bytes < need || reinterpret_cast<uintptr_t>(a->workspace) % 256 != 0)
             return FA_ERR_WORKSPACE;
         delta = static_cast<float*>(a->workspace);
         partials = reinterpret_cast<float*>(static_cast<char*>(a->workspace) + align256(delta_floats(p) * sizeof(float)));
+        if (dq_share_bytes(p) > 0) {
+            const FwdSplit s = fwd_split(p);
+            dq_splits = s.n_splits;
+            dq_keys = s.keys_per_split;
+            part_dq = reinterpret_cast<char*>(partials) + align256(partial_floats(p) * sizeof(float));
+        }
     } else {
         partials = delta + FA_NOALLOC_MAX_ROWS;
     }
@@ -322,6 +336,7 @@ int bwd_enqueue(const fa_bwd_args* a, void* stream, int stages, float* delta) {
     k.dq = a->dq; k.dk = a->dk; k.dv = a->dv; k.dbias = a->dbias;
     k.delta = delta;
     k.partials = partials;
+    k.dq_splits = dq_splits; k.dq_keys_per_split = dq_keys; k.part_dq = part_dq;
     k.sq = s3(a->q_strides); k.sk = s3(a->k_strides); k.sv = s3(a->v_strides); k.so = s3(a->o_strides);
     k.sdo = s3(a->do_strides); k.sdq = s3(a->dq_strides); k.sdk = s3(a->dk_strides); k.sdv = s3(a->dv_strides);
     if (a->bias && p.bias_dtype != FA_BIAS_ALIBI) {

@@ -73,25 +73,32 @@ __global__ __launch_bounds__(256, (StreamCfg<D, stream_kind(BIAS)>::MIN_BLOCKS))
     const int r = lane & 31, g = lane >> 5;
 
     int mt, bh;
-    decode_block<CAUSAL>(blockIdx.x, p.n_mtiles, p.B * p.H, mt, bh);
+    decode_block<CAUSAL>(blockIdx.x, p.n_mtiles * p.dq_splits, p.B * p.H, mt, bh);
+    // With the keys split between work-groups (never when causal) this one sees keys key0 ..
+    // key0 + N - 1 as if they were all there are (its dq is a share, summed afterwards); only ALiBi
+    // needs to know better.
+    const int split = mt % p.dq_splits;
+    mt /= p.dq_splits;
+    const int key0 = split * p.dq_keys_per_split;
     if (CAUSAL) mt = p.n_mtiles - 1 - mt;  // longest rows first
     const int b = bh / p.H, h = bh % p.H;
-    const int M = p.M, N = p.N;
+    const int M = p.M;
+    const int N = p.dq_splits > 1 ? (p.N - key0 < p.dq_keys_per_split ? p.N - key0 : p.dq_keys_per_split) : p.N;
     const int m0 = mt * BM;
     const int mw = m0 + wave * 32;  // first query row of this wave
     const int my_m = mw + r;
 
     const T* qp = reinterpret_cast<const T*>(p.q) + (int64_t)b * p.sq.b + (int64_t)h * p.sq.h;
-    const T* kp = reinterpret_cast<const T*>(p.k) + (int64_t)b * p.sk.b + (int64_t)h * p.sk.h;
-    const T* vp = reinterpret_cast<const T*>(p.v) + (int64_t)b * p.sv.b + (int64_t)h * p.sv.h;
+    const T* kp = reinterpret_cast<const T*>(p.k) + (int64_t)b * p.sk.b + (int64_t)h * p.sk.h + (int64_t)key0 * p.sk.s;
+    const T* vp = reinterpret_cast<const T*>(p.v) + (int64_t)b * p.sv.b + (int64_t)h * p.sv.h + (int64_t)key0 * p.sv.s;
     const E* bp = nullptr;
-    if (TB != 0) bp = reinterpret_cast<const E*>(p.bias) + (int64_t)b * p.sbias.b + (int64_t)h * p.sbias.h;
+    if (TB != 0) bp = reinterpret_cast<const E*>(p.bias) + (int64_t)b * p.sbias.b + (int64_t)h * p.sbias.h + (int64_t)key0 * p.sbias.n;
     float neg_slope = 0.f, ratio = 0.f;  // ALiBi: slope of this head, key positions per query row
     if (BIAS == 5) {
         neg_slope = -reinterpret_cast<const float*>(p.bias)[h];
         ratio = (float)p.N / (float)p.M;
     }
-    if (FROM_DS) bp = reinterpret_cast<const E*>(p.dbias) + (int64_t)b * p.sdbias.b + (int64_t)h * p.sdbias.h;
+    if (FROM_DS) bp = reinterpret_cast<const E*>(p.dbias) + (int64_t)b * p.sdbias.b + (int64_t)h * p.sdbias.h + (int64_t)key0 * p.sdbias.n;
 
     // Q^T and dO^T as B operands: column my_m, k = d
     const T* dop = reinterpret_cast<const T*>(p.dout) + (int64_t)b * p.sdo.b + (int64_t)h * p.sdo.h;
@@ -224,7 +231,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, stream_kind(BIAS)>::MIN_BLOCKS))
                     } else if constexpr (BIAS == 5) {
 #pragma unroll
                         for (int e = 0; e < 4; e++)
-                            bv[e] = alibi_bias(neg_slope, ratio, (float)my_m, (float)(n0 + nh + 4 * g) + (float)(8 * q4 + e));
+                            bv[e] = alibi_bias(neg_slope, ratio, (float)my_m, (float)(key0 + n0 + nh + 4 * g) + (float)(8 * q4 + e));
                     }
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
@@ -303,11 +310,39 @@ __global__ __launch_bounds__(256, (StreamCfg<D, stream_kind(BIAS)>::MIN_BLOCKS))
         }
     }
     __syncthreads();
-    T* op = reinterpret_cast<T*>(p.dq) + (int64_t)b * p.sdq.b + (int64_t)h * p.sdq.h;
+    const bool shared = p.dq_splits > 1;  // one of several shares of the keys: into this share's slice of the scratch
+    T* op = shared ? reinterpret_cast<T*>(p.part_dq) + ((int64_t)split * p.B * p.H + bh) * M * D
+                   : reinterpret_cast<T*>(p.dq) + (int64_t)b * p.sdq.b + (int64_t)h * p.sdq.h;
+    const int64_t o_stride = shared ? D : p.sdq.s;
     for (int c = lane; c < 32 * CPR; c += 64) {
         int row = c / CPR, ch = c % CPR;
-        if (mw + row < M) gst16(op + (int64_t)(mw + row) * p.sdq.s + ch * 8, lds_read16(o_lds + row * OS + ch * 8));
+        if (mw + row < M) gst16(op + (int64_t)(mw + row) * o_stride + ch * 8, lds_read16(o_lds + row * OS + ch * 8));
     }
+}
+
+// dq = sum of the shares that the work-groups of a split dQ kernel left in part_dq, added in fp32 in
+// a fixed order.  One thread per 8 head-dim elements of a row.
+template <typename T, int D> __global__ __launch_bounds__(256) void fa_bwd_dq_sum_kernel(const BwdParams p) {
+    typedef typename VecOf<T>::v8 T8;
+    constexpr int TPR = D / 8;
+    const int64_t rows = (int64_t)p.B * p.H * p.M;
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t row = idx / TPR;
+    const int c = (int)(idx % TPR);
+    if (row >= rows) return;
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < p.dq_splits; s++) {
+        const T8 v = as_vec<T8>(gld16(reinterpret_cast<const T*>(p.part_dq) + (s * rows + row) * D + c * 8));
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc[e] += (float)v[e];
+    }
+    const int m = (int)(row % p.M);
+    const int64_t bh = row / p.M;
+    const int b = (int)(bh / p.H), h = (int)(bh % p.H);
+    T8 o8;
+#pragma unroll
+    for (int e = 0; e < 8; e++) o8[e] = (T)acc[e];
+    gst16(reinterpret_cast<T*>(p.dq) + (int64_t)b * p.sdq.b + (int64_t)h * p.sdq.h + (int64_t)m * p.sdq.s + c * 8, as_raw(o8));
 }
 
 
@@ -1114,26 +1149,27 @@ template <typename T, int D> static hipError_t launch_all(const BwdParams& p, in
         }
     }
     if (stages & 4) {
-        dim3 qgrid((unsigned)(p.n_mtiles * p.B * p.H));
         // dBias in fp32 or in the element type of q, written densely a moment ago by the key-tile kernel
         // in rows of whole 16-byte chunks, is the dS the dQ product needs.  Only when that kernel ran in
         // this very call (or the caller vouches for the contents of dbias, bit 8) is it read.
         constexpr int DS_BIAS = __is_same(T, _Float16) ? 2 : 3;
         const bool ds_valid = dbias == 1 && ((stages & 2) || (stages & 8));
+        const bool from_ds = ds_valid && (bias == DS_BIAS || bias == 4) && p.dbias_vec;
+        // the one-product form runs at the rate of the dS stream and gains nothing from more work-groups
+        BwdParams pq = p;
+        if (from_ds) pq.dq_splits = 1;
+        dim3 qgrid((unsigned)(pq.n_mtiles * pq.dq_splits * pq.B * pq.H));
         if (ds_valid && bias == DS_BIAS && p.dbias_vec) {
-            if (causal) hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, DS_BIAS, true, true>), qgrid, dim3(256), 0, st, p);
-            else hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, DS_BIAS, false, true>), qgrid, dim3(256), 0, st, p);
-            return hipGetLastError();
-        }
-        if (ds_valid && bias == 4 && p.dbias_vec) {
-            if (causal) hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, 4, true, true>), qgrid, dim3(256), 0, st, p);
-            else hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, 4, false, true>), qgrid, dim3(256), 0, st, p);
-            return hipGetLastError();
-        }
+            if (causal) hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, DS_BIAS, true, true>), qgrid, dim3(256), 0, st, pq);
+            else hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, DS_BIAS, false, true>), qgrid, dim3(256), 0, st, pq);
+        } else if (ds_valid && bias == 4 && p.dbias_vec) {
+            if (causal) hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, 4, true, true>), qgrid, dim3(256), 0, st, pq);
+            else hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, 4, false, true>), qgrid, dim3(256), 0, st, pq);
+        } else {
 #define FA_CASE(BK)                                                                                               \
     case BK:                                                                                                      \
-        if (causal) hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, BK, true>), qgrid, dim3(256), 0, st, p);           \
-        else hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, BK, false>), qgrid, dim3(256), 0, st, p);                 \
+        if (causal) hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, BK, true>), qgrid, dim3(256), 0, st, pq);           \
+        else hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, BK, false>), qgrid, dim3(256), 0, st, pq);                 \
         break;
         switch (bias) {
             FA_CASE(0)
@@ -1145,7 +1181,13 @@ template <typename T, int D> static hipError_t launch_all(const BwdParams& p, in
             default: return hipErrorInvalidValue;
         }
 #undef FA_CASE
+        }
         e = hipGetLastError();
+        if (e == hipSuccess && pq.dq_splits > 1) {
+            const int64_t threads = (int64_t)p.B * p.H * p.M * (D / 8);
+            hipLaunchKernelGGL((fa_bwd_dq_sum_kernel<T, D>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, pq);
+            e = hipGetLastError();
+        }
     }
     return e;
 }

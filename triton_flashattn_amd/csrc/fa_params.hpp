@@ -57,6 +57,11 @@ struct BwdParams {
     int n_mtiles;   // query tiles of the dQ kernel
     int bias_vec;   // bias rows may be read with aligned 16-byte loads
     int dbias_vec;  // dbias rows may be written with aligned 16-byte stores
+    // dQ kernel: keys split between dq_splits work-groups per query tile (1 = no split), each over
+    // dq_keys_per_split keys, their shares of dq in the element type of q in part_dq (dq_splits,
+    // B*H, M, D); fa_bwd_dq_sum_kernel adds them up
+    int dq_splits, dq_keys_per_split;
+    void* part_dq;
     int row_bias_kind;  // 0, or the element kind (1 bool, 2 fp16, 3 bf16, 4 fp32) of a bias with stride 0 along M
                         // that the dK/dV kernel reads as one value per key
 };

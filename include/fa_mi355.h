@@ -126,7 +126,7 @@ size_t fa_bwd_workspace_bytes(const fa_problem *p);
 /* Scratch with which fa_fwd splits the keys of a query tile between several work-groups and merges
  * their softmaxes (the outputs of the shares in the element type of q, and their LSEs); 0 when the
  * problem has enough query tiles to fill the GPU, or is causal.  No counterpart in the reference (its grid is one program
- * per query tile, flash_attention.py:668).  The workspace is optional: without it fa_fwd runs one
+ * per query tile, flash_attention.py:666).  The workspace is optional: without it fa_fwd runs one
  * work-group per query tile, with the same results up to fp32 rounding of the merge. */
 size_t fa_fwd_workspace_bytes(const fa_problem *p);
 

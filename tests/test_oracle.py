@@ -201,3 +201,35 @@ def test_golden_fixtures_match_oracle():
         for name in ("out", "dq", "dk", "dv", "dbias"):
             if z[name] is not None:
                 assert torch.allclose(ref[name], z[name], atol=1e-5, rtol=1e-5), (f, name)
+
+
+def test_size_of_the_host_side_bias_rounding_that_is_not_restated():
+    """The reference multiplies a float bias by log2(e) in the bias dtype before its kernels see it
+    (flash_attention.py:663,704).  The default oracle (and the kernels) form that product in fp32.
+    HOST_ROUNDING restates the reference; this test records how far the two are apart: nothing for
+    an fp32 bias, below the parity tolerance for a bf16 bias of ordinary size and for a bf16 ALiBi
+    bias (large only where the softmax weight is negligible), far above it for a bf16 bias that is
+    large where the weight is (an offset of 1000 on every entry), where parity is therefore unpinned."""
+    import oracle.attention_oracle as orc
+    g = torch.Generator().manual_seed(3)
+    B, M, N, H, D = 1, 64, 4096, 2, 32
+    q, k, v = (torch.randn(B, n, H, D, generator=g).bfloat16() for n in (M, N, N))
+
+    def gap(bias):
+        a, _ = attention_forward(q, k, v, bias)
+        orc.HOST_ROUNDING = True
+        try:
+            b, _ = attention_forward(q, k, v, bias)
+        finally:
+            orc.HOST_ROUNDING = False
+        return (a - b).abs().max().item()
+
+    small = torch.randn(B, H, M, N, generator=g)
+    assert gap(small) < 1e-6                                   # fp32 bias: the same product
+    assert gap(small.bfloat16()) < 5e-3                        # |bias| of order 1 in bf16
+    i, j = torch.arange(M)[:, None].float(), torch.arange(N)[None, :].float()
+    slopes = torch.tensor([0.5, 0.0625])
+    alibi = (-slopes[:, None, None] * (i * N / M - j).abs())[None].bfloat16()   # down to -2048
+    assert alibi.float().abs().max() > 1000
+    assert gap(alibi) < 2e-2                                   # the large entries carry no weight
+    assert gap((small + 1000.0).bfloat16()) > 5e-2             # bf16 steps of 4 .. 8 on every entry: unpinned

@@ -47,7 +47,7 @@ static hipError_t launch_bwd(const BwdParams& p, int D, int dtype, int bias, boo
 }
 // query rows per work-group of the forward and dQ kernels; keys per work-group of the dK/dV kernel
 static int fwd_block_m() { return 128; }
-static int bwd_block_n(int) { return 128; }
+static int bwd_block_n(int D) { return D > 128 ? 64 : 128; }  // keys per tile of the dK/dV kernel
 }  // namespace fa
 
 // Scratch of fa_bwd_noalloc: delta, one float per (batch, head, query row), in the first half; the
@@ -163,7 +163,7 @@ void note_slow_bias(const char* what, const void* ptr, const int64_t s[4], const
 // dbias (column sums per (batch, head, key), or slope gradients per (batch, head, key tile, wave))
 size_t delta_floats(const fa_problem& p) { return (size_t)p.B * p.H * p.M; }
 size_t partial_floats(const fa_problem& p) {
-    const size_t tiles4 = (size_t)((p.N + fa::bwd_block_n(p.D) - 1) / fa::bwd_block_n(p.D)) * 4;
+    const size_t tiles4 = (size_t)((p.N + fa::bwd_block_n(p.D) - 1) / fa::bwd_block_n(p.D)) * (fa::bwd_block_n(p.D) / 32);
     return (size_t)p.B * p.H * ((size_t)p.N > tiles4 ? (size_t)p.N : tiles4);
 }
 
@@ -356,6 +356,7 @@ int bwd_enqueue(const fa_bwd_args* a, void* stream, int stages, float* delta) {
     int bn = fa::bwd_block_n(p.D);
     if (bn <= 0) return FA_ERR_UNSUPPORTED;
     k.n_ntiles = (p.N + bn - 1) / bn;
+    k.waves_per_role = bn / 32;
     k.n_mtiles = (p.M + fa::fwd_block_m() - 1) / fa::fwd_block_m();
     hipError_t e = fa::launch_bwd(k, p.D, p.dtype, p.bias_dtype, p.causal != 0, db_mode, stages,
                                   static_cast<hipStream_t>(stream));

@@ -403,7 +403,10 @@ constexpr bool bwd_occ2(int D, int bias) {
 #endif
 }
 template <int D, int BIAS, bool OCC2 = false> struct BwdCfg {
-    static constexpr int BN = 128, NT = 512;
+    // waves per role: four pairs of waves on a 128-key tile, two on a 64-key tile for head dim 256,
+    // where a wave needs the whole register file of its SIMD (two accumulator sets of 128 registers)
+    static constexpr int WPR = D > 128 ? 2 : 4;
+    static constexpr int BN = 32 * WPR, NT = 128 * WPR;
     static constexpr int LDS_LIMIT = OCC2 ? 81920 : 163840;
     static constexpr int NSUB = (D <= 64 && BIAS == 0 && !OCC2) ? 2 : 1;  // 32-row sub-blocks of a query block
     static constexpr int BMI = 32 * NSUB;
@@ -418,19 +421,19 @@ template <int D, int BIAS, bool OCC2 = false> struct BwdCfg {
     static constexpr int BCH = (BMI * BCPR + 63) / 64;     // bias copies per S-wave per block
     static constexpr int Q_BYTES = BMI * D * 2;
     static constexpr int NQD = Q_BYTES / 1024;             // 1 KB copies per Q (or dO) block
-    static constexpr int QD = NQD >= 4 ? NQD / 4 : 1;      // of which each wave of a role issues this many
+    static constexpr int QD = NQD >= WPR ? NQD / WPR : 1;  // of which each wave of a role issues this many
     // Q, dO, LSE, delta and the bias slices reach LDS through direct global -> LDS copies issued
     // LA blocks ahead of their use (Q, LSE and bias by the S-waves, dO and delta by the dP-waves);
     // a copy has LA - 1 whole steps and the rest of its own to land before the barrier that
     // publishes it.
     static constexpr int DS_BYTES = (BIAS == 2 || BIAS == 3) ? BN * DSS * 2 : 0;  // dS^T tiles (dBias)
-    static constexpr int P_BYTES = 4 * NSUB * 64 * 64;     // P hand-off: 16 floats per lane per sub-block
+    static constexpr int P_BYTES = 4 * NSUB * 64 * 16 * WPR;  // P hand-off: 16 floats per lane per sub-block
     static constexpr int BT_BYTES = BMI * 32 * ES;         // bias slice of one S-wave
     // LDS bytes with copies la blocks ahead: la + 1 dO buffers and bias slots, la + 2 Q buffers and
     // one more if the dK product of a block is deferred by a step (so that it does not wait for
     // the dS of the same step)
     static constexpr int lds_total(int la, int defer) {
-        return (2 * la + 3 + defer) * (Q_BYTES + BMI * 4) + DS_BYTES + 2 * P_BYTES + 4 * (la + 1) * BT_BYTES;
+        return (2 * la + 3 + defer) * (Q_BYTES + BMI * 4) + DS_BYTES + 2 * P_BYTES + WPR * (la + 1) * BT_BYTES;
     }
     static constexpr int LA = D > 128 ? 1 : (lds_total(3, 1) <= LDS_LIMIT ? 3 : 2);
     static constexpr bool DEFER_DK = D <= 128 && lds_total(LA, 1) <= LDS_LIMIT;
@@ -443,14 +446,15 @@ template <int D, int BIAS, bool OCC2 = false> struct BwdCfg {
     static constexpr int OFF_LSE = OFF_P + 2 * P_BYTES;
     static constexpr int OFF_DELTA = OFF_LSE + NQB * BMI * 4;
     static constexpr int OFF_BIAS = OFF_DELTA + NDOB * BMI * 4;
-    static constexpr int LOOP_BYTES = OFF_BIAS + 4 * RING * BT_BYTES;
+    static constexpr int LOOP_BYTES = OFF_BIAS + WPR * RING * BT_BYTES;
     static constexpr int LDS_BYTES = LOOP_BYTES;
     static_assert(LDS_BYTES <= LDS_LIMIT, "LDS budget of the configuration");
-    static constexpr int WAVES_PER_SIMD = OCC2 ? 4 : 2;
+    static constexpr int WAVES_PER_SIMD = OCC2 ? 4 : (WPR == 2 ? 1 : 2);
 };
 
 // Work split inside a work-group of 8 waves.  Waves 0-3 ("S-waves") and waves 4-7 ("dP-waves")
-// pair up on the four 32-key blocks of the tile (waves w and w + 4 run on the same SIMD):
+// pair up on the four 32-key blocks of the tile (waves w and w + 4 run on the same SIMD; for head
+// dim 256 a work-group is two such pairs on a 64-key tile, one wave per SIMD):
 //   S-wave : S = Q K^T, P = 2^(S*scale + bias - LSE)  -> hands P to its partner through LDS,
 //            dV^T += dO^T P, and the global -> LDS copies of the Q / LSE / bias blocks
 //   dP-wave: dP = dO V^T, dS = P (dP - delta) (+ dBias through an LDS tile), dK^T += Q^T dS,
@@ -465,7 +469,7 @@ template <int D, int BIAS, bool OCC2 = false> struct BwdCfg {
 // query rows, one fp32 per (batch, head, key), for ALiBi the gradient of the slope, one fp32 per
 // (batch, head, key tile, wave); a second small kernel sums those over the broadcast dimensions.
 template <typename T, int D, int BIAS, bool CAUSAL, int DBIAS>
-__global__ __launch_bounds__(512, (BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>::WAVES_PER_SIMD)) void fa_bwd_kernel(const BwdParams p) {
+__global__ __launch_bounds__((BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>::NT), (BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>::WAVES_PER_SIMD)) void fa_bwd_kernel(const BwdParams p) {
     constexpr int TB = tile_kind(BIAS);  // kind of bias tile that is streamed (none for ALiBi)
     typedef BwdCfg<D, TB, bwd_occ2(D, BIAS)> C;
     typedef Swz<D> SW;
@@ -481,8 +485,8 @@ __global__ __launch_bounds__(512, (BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
     const int r = lane & 31, g = lane >> 5;
-    const bool s_wave = wave < 4;  // role
-    const int kb = __builtin_amdgcn_readfirstlane(wave & 3);  // 32-key block of this wave (scalar)
+    const bool s_wave = wave < C::WPR;  // role
+    const int kb = __builtin_amdgcn_readfirstlane(wave % C::WPR);  // 32-key block of this wave (scalar)
     const unsigned lds_base = lds_addr_of(smem);
 
     int nt, bh;
@@ -1029,7 +1033,7 @@ __global__ __launch_bounds__(512, (BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>
                 float s = red_acc;
 #pragma unroll
                 for (int w = 32; w >= 1; w >>= 1) s += __shfl_xor(s, w, 64);
-                if (lane == 0) p.partials[((int64_t)bh * p.n_ntiles + nt) * 4 + kb] = s;
+                if (lane == 0) p.partials[((int64_t)bh * p.n_ntiles + nt) * C::WPR + kb] = s;
             } else {
                 // column sums: lanes l and l + 32 hold different rows of the same key
                 const float s = pair_sum(red_acc);
@@ -1062,7 +1066,7 @@ __global__ __launch_bounds__(512, (BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>
 template <typename T, int D, int BIAS, bool CAUSAL, int DBIAS>
 static hipError_t launch_main(const BwdParams& p, hipStream_t st) {
     dim3 grid((unsigned)(p.n_ntiles * p.B * p.H));
-    hipLaunchKernelGGL((fa_bwd_kernel<T, D, BIAS, CAUSAL, DBIAS>), grid, dim3(512), 0, st, p);
+    hipLaunchKernelGGL((fa_bwd_kernel<T, D, BIAS, CAUSAL, DBIAS>), grid, dim3((BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>::NT)), 0, st, p);
     return hipGetLastError();
 }
 
@@ -1089,7 +1093,7 @@ template <int LANES>
 __global__ __launch_bounds__(LANES) void fa_bwd_slope_reduce_kernel(const BwdParams p) {
     static_assert(LANES == 64, "one wave");
     const int h = blockIdx.x, lane = threadIdx.x;
-    const int per_bh = p.n_ntiles * 4;
+    const int per_bh = p.n_ntiles * p.waves_per_role;
     float s = 0.f;
     for (int b = 0; b < p.B; b++)
         for (int i = lane; i < per_bh; i += 64) s += p.partials[((int64_t)b * p.H + h) * per_bh + i];

@@ -54,6 +54,7 @@ struct BwdParams {
     int B, H, M, N;
     float sm_scale;
     int n_ntiles;   // key tiles of the dK/dV kernel
+    int waves_per_role;  // 32-key blocks per key tile of the dK/dV kernel
     int n_mtiles;   // query tiles of the dQ kernel
     int bias_vec;   // bias rows may be read with aligned 16-byte loads
     int dbias_vec;  // dbias rows may be written with aligned 16-byte stores

@@ -279,7 +279,11 @@ __global__ __launch_bounds__(256, (StreamCfg<D, stream_kind(BIAS)>::MIN_BLOCKS))
     // one of several shares of the keys: output and LSE go to this share's slice of the scratch
     const bool shared = p.n_splits > 1;
     float* lse_out = shared ? p.part_lse + ((int64_t)split * p.B * p.H + bh) * M : p.lse + ((int64_t)b * p.H + h) * M;
-    if (g == 0 && my_m < M) lse_out[my_m] = m_i + fast_log2(l_tot);
+    // (the row index passes through an empty asm so that the store address is formed here and not
+    // kept in two registers across the loops)
+    int my_m_late = my_m;
+    asm volatile("" : "+v"(my_m_late));
+    if (g == 0 && my_m_late < M) lse_out[my_m_late] = m_i + fast_log2(l_tot);
 
     ks_.drain();  // K/V slots are dead and no copy is in flight: reuse their LDS for the output tile
     T* o_lds = reinterpret_cast<T*>(smem) + wave * 32 * OS;

@@ -394,17 +394,13 @@ template <> struct BiasQuad<4> {
 
 // ---------------------------------------------------------------------------------------------
 // OCC2: two work-groups per CU (four waves per SIMD, 128 registers each, half of the LDS): the
-// configuration of the small head dims without a float bias, whose blocks are small enough.
-constexpr bool bwd_occ2(int D, int bias) {
-#ifdef FA_EXP_NO_OCC2
-    return false;
-#else
-    return D <= 64 && (bias == 0 || bias == 6 || bias == 7);
-#endif
-}
+// configuration of the small head dims without a bias tile (no bias, or one kept in a register per
+// key), whose blocks are small enough.
+constexpr bool bwd_occ2(int D, int bias) { return D <= 64 && (bias == 0 || bias == 6 || bias == 7); }
 template <int D, int BIAS, bool OCC2 = false> struct BwdCfg {
     // waves per role: four pairs of waves on a 128-key tile, two on a 64-key tile for head dim 256,
-    // where a wave needs the whole register file of its SIMD (two accumulator sets of 128 registers)
+    // where a wave needs the whole register file of its SIMD (128 accumulator registers and 64 of the
+    // resident operand before anything streams)
     static constexpr int WPR = D > 128 ? 2 : 4;
     static constexpr int BN = 32 * WPR, NT = 128 * WPR;
     static constexpr int LDS_LIMIT = OCC2 ? 81920 : 163840;

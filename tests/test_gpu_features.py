@@ -38,8 +38,13 @@ def test_alibi_matches_oracle_on_the_materialised_bias(gpu_device, D, causal):
         check(ours, ref, "alibi D%d %s" % (D, (B, M, N, H)))
         dist = dense / slopes.detach().view(1, H, 1, 1)          # -|i N / M - j|
         want = (ref["dbias"] * dist).sum(dim=(0, 2, 3))
+        # the slope gradient is a sum of M N signed terms that cancel to a small part of their total
+        # size; the error of 16-bit arithmetic (delta is formed from the rounded output, as in the
+        # reference, flash_attention.py:215-227, which shifts every dS of a row the same way) scales
+        # with that size, not with the sum: 2^-8 of it for bf16
+        size = (ref["dbias"] * dist).abs().sum(dim=(0, 2, 3))
         assert slopes.grad.shape == (H,)
-        assert rel_l2(slopes.grad, want) <= GRAD_RTOL, (D, B, M, N, H, slopes.grad, want)
+        assert ((slopes.grad - want).abs() <= 5e-3 * size + 1e-6).all(), (D, B, M, N, H, slopes.grad, want, size)
 
 
 def test_alibi_is_deterministic_and_needs_no_gradient(gpu_device):

@@ -113,6 +113,36 @@ def test_row_broadcast_bias_never_becomes_dense(gpu_device):
         assert torch.isfinite(ours["dq"].float()).all()
 
 
+@pytest.mark.parametrize("D", [16, 64, 128, 256])
+@pytest.mark.parametrize("kind", ["bool", "f16", "bf16", "f32"])
+def test_row_broadcast_bias_is_staged_once_per_work_group(gpu_device, D, kind):
+    """The forward and dQ kernels keep a bias without a row dimension as an fp32 row in LDS (up to
+    4096 keys per work-group): every element kind, ragged and causal shapes, a strided row, a row that
+    is split between work-groups, one that is too long for LDS (dense path through the zero stride),
+    and a batch whose keys are all masked."""
+    bdt = {"bool": torch.bool, "f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}[kind]
+    cases = [  # B, M, N, H, causal, key stride of the bias row
+        (2, 300, 333, 3, False, 1), (2, 333, 333, 2, True, 1), (1, 130, 1000, 2, False, 2),
+        (1, 64, 4096, 2, False, 1), (1, 40, 4200, 1, False, 1), (1, 96, 6000, 2, False, 1)]
+    for i, (B, M, N, H, causal, step) in enumerate(cases):
+        q, k, v, do, _ = make_inputs(gpu_device, B, M, N, H, D, torch.bfloat16 if i % 2 else torch.float16, None, seed=7 * D + i)
+        g = torch.Generator().manual_seed(100 + i)
+        if kind == "bool":
+            row = torch.rand(B, 1, 1, N * step, generator=g) < 0.7
+            if B > 1:
+                row[1] = False  # every key of batch 1 masked: uniform attention (flash_attention.py:49-53)
+            bias = row.to(gpu_device)[..., ::step]
+        else:
+            bias = torch.randn(1, H, 1, N * step, generator=g).to(bdt).to(gpu_device)[..., ::step].requires_grad_(True)
+        assert bias.stride(-1) == step
+        ours = run_ours(q, k, v, do, bias, causal)
+        full = bias.detach().broadcast_to(B, H, M, N)
+        ref = run_oracle(q, k, v, do, full if kind == "bool" else full.float(), causal)
+        if kind != "bool":
+            ref["dbias"] = ref["dbias"].sum_to_size(1, H, 1, N)
+        check(ours, ref, "D%d %s case %d" % (D, kind, i))
+
+
 def test_batch_or_head_broadcast_bias(gpu_device):
     """A bias broadcast over batches or heads only keeps its (M, N) tiles: read through an expanded
     view, gradient computed densely and summed over the broadcast dimensions."""

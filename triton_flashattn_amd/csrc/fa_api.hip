@@ -183,7 +183,7 @@ FwdSplit fwd_split(const fa_problem& p) {
     s = s > 4 ? 4 : s;
     while (s > 1 && n_steps / s < 16) s--;
     if (s <= 1) return {1, 0};
-    return {s, (n_steps + s - 1) / s * bk};
+    return {s, ((n_steps + s - 1) / s * bk + 63) / 64 * 64};  // whole steps of either kernel tiling
 }
 
 // the shares of dq of a dQ kernel that splits its keys like the forward (0 when it does not)
@@ -275,6 +275,10 @@ int fa_fwd(const fa_fwd_args* a, void* stream) {
             k.part_lse = reinterpret_cast<float*>(static_cast<char*>(a->workspace) + align256((size_t)s.n_splits * rows * p.D * 2));
         }
     }
+    // a bias that does not depend on the query row and whose keys fit the kernel's LDS row
+    if (a->bias && p.bias_dtype >= FA_BIAS_BOOL && p.bias_dtype <= FA_BIAS_F32 && (p.M == 1 || a->bias_strides[2] == 0) &&
+        (k.n_splits > 1 ? k.keys_per_split : p.N) <= fa::kRowBiasKeys)
+        k.row_bias_kind = p.bias_dtype;
     hipError_t e = fa::launch_fwd(k, p.D, p.dtype, p.bias_dtype, p.causal != 0, static_cast<hipStream_t>(stream));
     if (e == hipErrorNotSupported) return FA_ERR_UNSUPPORTED;
     return e == hipSuccess ? FA_OK : FA_ERR_LAUNCH;

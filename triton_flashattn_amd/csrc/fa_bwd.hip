@@ -65,8 +65,12 @@ __global__ __launch_bounds__(256, (StreamCfg<D, stream_kind(BIAS)>::MIN_BLOCKS))
     typedef typename VecOf<T>::v4 T4;
     typedef typename BiasElem<tile_kind(BIAS)>::type E;
     constexpr int BM = C::BM, BK = C::BK, OS = C::OS, CPR = C::CPR;
+    constexpr bool ROWB = BIAS >= 6;     // the same bias for every query row, kept as an fp32 row in LDS
+    constexpr bool BOOLROW = BIAS == 7;  // ... a bool mask: the row holds 0 or the mask term, in log2 units
+    static_assert(!(FROM_DS && ROWB), "a row-broadcast bias has no dense dS");
 
-    __shared__ __align__(1024) unsigned char smem[C::LDS_BYTES];
+    __shared__ __align__(1024) unsigned char smem[C::LDS_BYTES + (ROWB ? kRowBiasKeys * 4 : 0)];
+    const float* row_lds = reinterpret_cast<const float*>(smem + C::LDS_BYTES);
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
@@ -99,6 +103,10 @@ __global__ __launch_bounds__(256, (StreamCfg<D, stream_kind(BIAS)>::MIN_BLOCKS))
         ratio = (float)p.N / (float)p.M;
     }
     if (FROM_DS) bp = reinterpret_cast<const E*>(p.dbias) + (int64_t)b * p.sdbias.b + (int64_t)h * p.sdbias.h + (int64_t)key0 * p.sdbias.n;
+
+    if (ROWB)
+        stage_row_bias(reinterpret_cast<float*>(smem + C::LDS_BYTES), p.bias, p.row_bias_kind,
+                       (int64_t)b * p.sbias.b + (int64_t)h * p.sbias.h + (int64_t)key0 * p.sbias.n, p.sbias.n, N, tid);
 
     // Q^T and dO^T as B operands: column my_m, k = d
     const T* dop = reinterpret_cast<const T*>(p.dout) + (int64_t)b * p.sdo.b + (int64_t)h * p.sdo.h;
@@ -232,6 +240,10 @@ __global__ __launch_bounds__(256, (StreamCfg<D, stream_kind(BIAS)>::MIN_BLOCKS))
 #pragma unroll
                         for (int e = 0; e < 4; e++)
                             bv[e] = alibi_bias(neg_slope, ratio, (float)my_m, (float)(key0 + n0 + nh + 4 * g) + (float)(8 * q4 + e));
+                    } else if constexpr (ROWB) {
+                        f32x4 w = *reinterpret_cast<const f32x4*>(row_lds + n0 + nh + nl);
+#pragma unroll
+                        for (int e = 0; e < 4; e++) bv[e] = w[e];
                     }
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
@@ -245,7 +257,8 @@ __global__ __launch_bounds__(256, (StreamCfg<D, stream_kind(BIAS)>::MIN_BLOCKS))
                             if (CAUSAL) t += (my_m < n) ? kMask : 0.f;
                             float add = 0.f;
                             if (BIAS == 1) add = keep[e] ? 0.f : kMask;
-                            if (BIAS >= 2) add = __fmul_rn(bv[e], kLog2e);
+                            if (BOOLROW) add = bv[e];
+                            if (BIAS >= 2 && !BOOLROW) add = __fmul_rn(bv[e], kLog2e);
                             if (BIAS != 0) add = oob ? kMask : add;  // out-of-range bias reads as masked
                             x = __fadd_rn(x, __fadd_rn(t, add));
                             pv = fast_exp2(x - lse_i);
@@ -253,6 +266,8 @@ __global__ __launch_bounds__(256, (StreamCfg<D, stream_kind(BIAS)>::MIN_BLOCKS))
                             pv = fast_exp2(__builtin_fmaf(s[i], qk_scale, -lse_i));
                         } else if constexpr (BIAS == 1) {
                             pv = fast_exp2(__builtin_fmaf(s[i], qk_scale, (keep[e] ? 0.f : kMask) - lse_i));
+                        } else if constexpr (BOOLROW) {
+                            pv = fast_exp2(__builtin_fmaf(s[i], qk_scale, bv[e] - lse_i));
                         } else {
                             pv = fast_exp2(__builtin_fmaf(bv[e], kLog2e, __builtin_fmaf(s[i], qk_scale, -lse_i)));
                         }
@@ -1171,13 +1186,19 @@ template <typename T, int D> static hipError_t launch_all(const BwdParams& p, in
         if (causal) hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, BK, true>), qgrid, dim3(256), 0, st, pq);           \
         else hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, BK, false>), qgrid, dim3(256), 0, st, pq);                 \
         break;
-        switch (bias) {
+        // a bias without a row dimension whose keys (of one share) fit the LDS row is staged once per
+        // work-group instead of streamed
+        const int keys_per_wg = pq.dq_splits > 1 ? pq.dq_keys_per_split : pq.N;
+        const int qbias = (p.row_bias_kind != 0 && keys_per_wg <= kRowBiasKeys) ? (p.row_bias_kind == 1 ? 7 : 6) : bias;
+        switch (qbias) {
             FA_CASE(0)
             FA_CASE(1)
             FA_CASE(2)
             FA_CASE(3)
             FA_CASE(4)
             FA_CASE(5)
+            FA_CASE(6)
+            FA_CASE(7)
             default: return hipErrorInvalidValue;
         }
 #undef FA_CASE

@@ -256,17 +256,43 @@ template <> struct BiasElem<7> { typedef unsigned char type; };
 // Bias kind 5 (ALiBi): bias[b,h,i,j] = -slope[h] * |i * N / M - j| is computed from the indices, so no
 // bias tile exists and the K/V stream is tiled as without a bias.  TILE_KIND maps a bias kind to
 // the kind of tile that StreamCfg / KeyStream handle.
-// Kinds 6 and 7 exist in the dK/dV kernel only: a float bias / a bool mask that is the same for every
-// query row (stride 0 along M).  There the lane is the key, so the whole bias of a wave is ONE
-// register per lane, read once, and nothing is streamed.
+// Kinds 6 and 7: a float bias / a bool mask that is the same for every query row (stride 0 along M).
+// In the dK/dV kernel the lane is the key, so the whole bias of a wave is ONE register per lane, read
+// once, and nothing is streamed.  In the forward and dQ kernels the lane is the row: the work-group
+// converts the row to fp32 once into an LDS region behind the K/V slots (at most kRowBiasKeys keys,
+// longer rows take the dense path through their zero stride) and every lane reads the values of its
+// keys from there; the K/V stream is tiled as without a bias.
 constexpr int tile_kind(int bias) { return bias >= 5 ? 0 : bias; }
 // ... and to the kind that StreamCfg / KeyStream tile the K/V stream for: 6 = no bias tile, but steps of
 // 32 keys like the kernels with one (the element-wise work of ALiBi needs the registers that the
 // 64-key steps of the bias-free kernels spend on a second block of scores)
-constexpr int stream_kind(int bias) { return bias == 5 ? 6 : bias; }
+constexpr int stream_kind(int bias) { return bias == 5 ? 6 : (bias >= 6 ? 0 : bias); }
 // -slope * |m * ratio - n| for query row m and key n (both exact as floats), natural units
 __device__ __forceinline__ float alibi_bias(float neg_slope, float ratio, float mf, float nf) {
     return neg_slope * __builtin_fabsf(__builtin_fmaf(mf, ratio, -nf));
+}
+
+// Kinds 6 / 7 of the forward and dQ kernels: the 256 threads of a work-group write the bias row of
+// keys 0 .. N-1 (element kind 1 bool, 2 fp16, 3 bf16, 4 fp32, n-th element at bias[at0 + n stride_n])
+// to row_lds as fp32, a float bias in natural units, a bool mask as the additive term of the
+// reference in log2 units (0 or -1e6, flash_attention.py:49-53); zeros up to the next multiple of 64.
+__device__ __forceinline__ void stage_row_bias(float* row_lds, const void* bias, int kind, int64_t at0, int64_t stride_n,
+                                               int N, int tid) {
+    const int n_stage = (N + 63) & ~63;
+    for (int n = tid; n < n_stage; n += 256) {
+        float v = 0.f;
+        if (n < N) {
+            const int64_t at = at0 + (int64_t)n * stride_n;
+            switch (kind) {
+                case 1: v = reinterpret_cast<const unsigned char*>(bias)[at] != 0 ? 0.f : kMask; break;
+                case 2: v = (float)reinterpret_cast<const _Float16*>(bias)[at]; break;
+                case 3: v = (float)reinterpret_cast<const __bf16*>(bias)[at]; break;
+                default: v = reinterpret_cast<const float*>(bias)[at]; break;
+            }
+        }
+        row_lds[n] = v;
+    }
+    __syncthreads();
 }
 
 // Tiling of the forward and the dQ kernel: a work-group owns 128 query rows (4 waves x 32 rows) and streams

@@ -26,17 +26,26 @@
 
 namespace fa {
 
+// The K/V stream of a row-broadcast bias (kinds 6, 7) is tiled like that of ALiBi, in steps of 32
+// keys: the bias values of a block need the registers that 64-key steps spend on a second block of
+// scores.
+constexpr int fwd_stream_kind(int bias) { return bias >= 5 ? 6 : bias; }
+
 template <typename T, int D, int BIAS, bool CAUSAL>
-__global__ __launch_bounds__(256, (StreamCfg<D, stream_kind(BIAS)>::MIN_BLOCKS)) void fa_fwd_kernel(const FwdParams p) {
+__global__ __launch_bounds__(256, (StreamCfg<D, fwd_stream_kind(BIAS)>::MIN_BLOCKS)) void fa_fwd_kernel(const FwdParams p) {
     constexpr int TB = tile_kind(BIAS);  // kind of bias tile that is streamed (none for ALiBi)
-    typedef StreamCfg<D, stream_kind(BIAS)> C;
+    typedef StreamCfg<D, fwd_stream_kind(BIAS)> C;
     typedef Swz<D> SW;
     typedef typename VecOf<T>::v8 T8;
     typedef typename VecOf<T>::v4 T4;
     typedef typename BiasElem<tile_kind(BIAS)>::type E;
     constexpr int BM = C::BM, BK = C::BK, OS = C::OS, CPR = C::CPR;
 
-    __shared__ __align__(1024) unsigned char smem[C::LDS_BYTES];
+    constexpr bool ROWB = BIAS >= 6;     // the same bias for every query row, kept as an fp32 row in LDS
+    constexpr bool BOOLROW = BIAS == 7;  // ... a bool mask: the row holds 0 or the mask term, in log2 units
+
+    __shared__ __align__(1024) unsigned char smem[C::LDS_BYTES + (ROWB ? kRowBiasKeys * 4 : 0)];
+    const float* row_lds = reinterpret_cast<const float*>(smem + C::LDS_BYTES);
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
@@ -69,6 +78,10 @@ __global__ __launch_bounds__(256, (StreamCfg<D, stream_kind(BIAS)>::MIN_BLOCKS))
         ratio = (float)p.N / (float)p.M;
     }
 
+    if (ROWB)
+        stage_row_bias(reinterpret_cast<float*>(smem + C::LDS_BYTES), p.bias, p.row_bias_kind,
+                       (int64_t)b * p.sbias.b + (int64_t)h * p.sbias.h + (int64_t)key0 * p.sbias.n, p.sbias.n, N, tid);
+
     // Q^T as B operand: column my_m, k = d
     T8 qreg[C::KSTEPS];
 #pragma unroll
@@ -93,7 +106,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, stream_kind(BIAS)>::MIN_BLOCKS))
         for (int i = 0; i < 16; i++) o_acc[db][i] = 0.f;
 
     const unsigned rows_l = SW::rows_lane(lane), cols_l = SW::cols_lane(lane);
-    KeyStream<T, D, stream_kind(BIAS)> ks_;
+    KeyStream<T, D, fwd_stream_kind(BIAS)> ks_;
     ks_.init(smem, kp, vp, bp, p.sk.s, p.sv.s, p.sbias.m, p.sbias.n, M, N, mw, wave, lane);
 
     // One step of the K/V stream.  Interior steps (every key in range and visible to every row of
@@ -184,6 +197,10 @@ __global__ __launch_bounds__(256, (StreamCfg<D, stream_kind(BIAS)>::MIN_BLOCKS))
                 } else if constexpr (BIAS == 5) {
 #pragma unroll
                     for (int e = 0; e < 4; e++) bv[e] = alibi_bias(neg_slope, ratio, mf, nf0 + (float)(8 * q4 + e));
+                } else if constexpr (ROWB) {
+                    f32x4 w = *reinterpret_cast<const f32x4*>(row_lds + n0 + nh + nl);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) bv[e] = w[e];
                 }
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
@@ -196,13 +213,16 @@ __global__ __launch_bounds__(256, (StreamCfg<D, stream_kind(BIAS)>::MIN_BLOCKS))
                         if (CAUSAL) t += (my_m < n) ? kMask : 0.f;
                         float add = 0.f;
                         if (BIAS == 1) add = keep[e] ? 0.f : kMask;
-                        if (BIAS >= 2) add = __fmul_rn(bv[e], kLog2e);
+                        if (BOOLROW) add = bv[e];
+                        if (BIAS >= 2 && !BOOLROW) add = __fmul_rn(bv[e], kLog2e);
                         if (BIAS != 0) add = (n >= N) ? kMask : add;  // out-of-range bias reads as masked
                         x = __fadd_rn(x, __fadd_rn(t, add));
                     } else if constexpr (BIAS == 0) {
                         x = s[i];                                    // raw score, scale folded below
                     } else if constexpr (BIAS == 1) {
                         x = keep[e] ? s[i] * qk_scale : s[i] * qk_scale + kMask;
+                    } else if constexpr (BOOLROW) {
+                        x = s[i] * qk_scale + bv[e];
                     } else {
                         x = s[i] * p.sm_scale + bv[e];               // natural units
                     }
@@ -212,7 +232,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, stream_kind(BIAS)>::MIN_BLOCKS))
             }
             // units of x: log2 (MASKED, bool bias), raw dot product (no bias), natural (float bias)
             constexpr bool RAW = !MASKED && BIAS == 0;
-            constexpr bool NAT = !MASKED && BIAS >= 2;
+            constexpr bool NAT = !MASKED && BIAS >= 2 && !BOOLROW;
             const float to_log2 = RAW ? qk_scale : (NAT ? kLog2e : 1.f);
             mx = pair_max(mx) * to_log2;
             const bool raise = mx > m_i + 8.f;
@@ -353,6 +373,8 @@ template <typename T, int D> static hipError_t launch_bias(const FwdParams& p, i
 #define FA_CASE(BK)                                                        \
     case BK:                                                               \
         return causal ? launch_one<T, D, BK, true>(p, st) : launch_one<T, D, BK, false>(p, st);
+    // a bias without a row dimension is staged once per work-group instead of streamed
+    if (p.row_bias_kind != 0) bias = p.row_bias_kind == 1 ? 7 : 6;
     switch (bias) {
         FA_CASE(0)
         FA_CASE(1)
@@ -360,6 +382,8 @@ template <typename T, int D> static hipError_t launch_bias(const FwdParams& p, i
         FA_CASE(3)
         FA_CASE(4)
         FA_CASE(5)
+        FA_CASE(6)
+        FA_CASE(7)
     }
 #undef FA_CASE
     return hipErrorInvalidValue;

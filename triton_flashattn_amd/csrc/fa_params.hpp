@@ -13,6 +13,9 @@ struct Strides4 {
     int64_t b, h, m, n;
 };
 
+// keys of a row-broadcast bias that the forward and dQ kernels keep in LDS (as fp32)
+constexpr int kRowBiasKeys = 4096;
+
 struct FwdParams {
     const void* q;
     const void* k;
@@ -33,6 +36,8 @@ struct FwdParams {
     int n_splits, keys_per_split;
     void* part_o;
     float* part_lse;
+    int row_bias_kind;  // 0, or the element kind (1 bool, 2 fp16, 3 bf16, 4 fp32) of a bias with stride 0 along M
+                        // whose keys (of one split) fit the kernel's LDS row: staged once, not streamed
 };
 
 struct BwdParams {
@@ -63,8 +68,8 @@ struct BwdParams {
     // B*H, M, D); fa_bwd_dq_sum_kernel adds them up
     int dq_splits, dq_keys_per_split;
     void* part_dq;
-    int row_bias_kind;  // 0, or the element kind (1 bool, 2 fp16, 3 bf16, 4 fp32) of a bias with stride 0 along M
-                        // that the dK/dV kernel reads as one value per key
+    int row_bias_kind;  // 0, or the element kind (1 bool, 2 fp16, 3 bf16, 4 fp32) of a bias with stride 0 along M:
+                        // the dK/dV kernel reads it as one value per key, the dQ kernel stages it in LDS
 };
 
 }  // namespace fa

@@ -17,9 +17,12 @@
  *   lse, delta   : (B, H, M) fp32, dense, in log2 units: lse = log2(sum_j 2^(s_ij))
  * Base pointers of q/k/v/o/do/dq/dk/dv and their B/seq/H strides must be multiples of 16 bytes
  * (FA_ERR_LAYOUT otherwise; FA_ERR_HEAD_STRIDE for a D stride other than 1); bias/dbias have no
- * alignment requirement, but rows with unit N stride and 16-byte aligned row starts take the fast
- * path.  With FA_MI355_VERBOSE set in the environment the library says on stderr, once per process,
- * when a bias or dbias misses that path and is read or written element by element.
+ * alignment requirement, but only rows with unit N stride and 16-byte aligned row starts that are
+ * whole 16-byte chunks, or whose row stride covers the last chunk (N * element size rounded up to 16
+ * bytes: a padded row pitch or a column slice of a wider tensor; the bytes behind the last key of
+ * every row are then read, never written), take the fast path.  With FA_MI355_VERBOSE set in the
+ * environment the library says on stderr, once per process, when a bias or dbias misses that path
+ * and is read or written element by element (several times slower).
  */
 #ifndef FA_MI355_H
 #define FA_MI355_H

@@ -216,7 +216,11 @@ def test_gradients_nobody_asks_for_are_skipped(gpu_device):
             t[n].requires_grad_(True)
         flash_attention_fn(t["q"], t["k"], t["v"], t["bias"]).backward(do)
         for n in ("q", "k", "v", "bias"):
-            if n in wanted:
+            if n in wanted and n == "q" and "bias" not in wanted:
+                # without a bias gradient there is no dS tensor to read: dq comes from the kernel
+                # that recomputes the scores, which rounds differently
+                assert rel_l2(t[n].grad, full["d" + n].float()) <= 1e-2, (wanted, n)
+            elif n in wanted:
                 assert torch.equal(t[n].grad, full["d" + n]), (wanted, n)
             else:
                 assert t[n].grad is None

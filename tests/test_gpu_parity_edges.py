@@ -170,3 +170,53 @@ def test_dq_routes_agree(gpu_device):
     assert rel_l2(slow[3], whole[3].float()) < 1e-3
     for i in (1, 2):
         assert rel_l2(slow[i], whole[i].float()) < 1e-2
+
+
+# ---------------------------------------------------------------- bias rows that are not whole 16-byte chunks
+def _launch_directly(q, k, v, do, bias, dbias, causal):
+    """The two launchers below the layer that pads bias rows: the kernels see `bias` and `dbias` as
+    they are.  Returns out, dq, dk, dv."""
+    sm_scale = q.shape[-1] ** -0.5
+    o, lse = _flash_attn_fwd(q, k, v, bias, causal, sm_scale)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    fa_mod._flash_attn_bwd(do, q, k, v, o, bias, causal, sm_scale, lse, dq, dk, dv, dbias)
+    return {"out": o, "dq": dq, "dk": dk, "dv": dv, "dbias": dbias}
+
+
+@pytest.mark.parametrize("D", [32, 128])
+@pytest.mark.parametrize("kind", ["bool", "f16", "bf16", "f32"])
+def test_bias_rows_that_are_not_whole_chunks(gpu_device, D, kind):
+    """A number of keys that is no multiple of 16 bytes, three ways: through the public function
+    (which copies such a bias into rows with a padded pitch), straight to the kernels as a dense
+    tensor (read and written element by element) and straight to the kernels as a column slice of a
+    wider tensor (16-byte copies that run into the columns behind the slice: those hold NaN for the
+    bias and must not be touched in dbias)."""
+    bdt = {"bool": torch.bool, "f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}[kind]
+    for i, (B, M, N, H, causal) in enumerate([(2, 70, 197, 2, False), (1, 131, 131, 3, True), (1, 257, 67, 1, False)]):
+        dtype = torch.float16 if kind == "f16" else torch.bfloat16
+        q, k, v, do, bias = make_inputs(gpu_device, B, M, N, H, D, dtype, kind, seed=11 * D + i, trainable=False)
+        assert (N * bias.element_size()) % 16 != 0
+        trainable = kind != "bool"
+        ref = run_oracle(q, k, v, do, bias, causal)
+        if not trainable:
+            ref["dbias"] = None
+        # the public function
+        leaf = bias.clone().requires_grad_(trainable)
+        ours = run_ours(q, k, v, do, leaf, causal)
+        check(ours, ref, "public %s D%d case %d" % (kind, D, i))
+        if trainable:
+            assert ours["dbias"].shape == bias.shape and ours["dbias"].dtype == bdt
+        # dense rows, element by element
+        dbias = torch.empty_like(bias) if trainable else None
+        check(_launch_directly(q, k, v, do, bias, dbias, causal), ref, "dense %s D%d case %d" % (kind, D, i))
+        # a column slice of a wider tensor
+        per = 16 // bias.element_size()
+        width = -(-N // per) * per + per * (i % 2)   # rows start at multiples of 16 bytes and own their last chunk
+        wide = torch.full((B, H, M, width), float("nan") if trainable else 1, dtype=bdt, device=gpu_device)
+        wide[..., :N] = bias
+        dwide = torch.full((B, H, M, width), 7.0, dtype=bdt, device=gpu_device) if trainable else None
+        assert fa_mod._bias_rows_ok(wide[..., :N]) and not fa_mod._bias_rows_ok(bias)
+        res = _launch_directly(q, k, v, do, wide[..., :N], None if dwide is None else dwide[..., :N], causal)
+        check(res, ref, "slice %s D%d case %d" % (kind, D, i))
+        if trainable:
+            assert (dwide[..., N:] == 7.0).all(), "the columns behind the dbias slice were written"

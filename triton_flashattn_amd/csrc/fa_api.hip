@@ -137,10 +137,14 @@ bool bias_vec_ok(const void* ptr, const int64_t s[4], const fa_problem& p) {
     if (p.B > 1 && (s[0] * es) % 16 != 0) return false;
     if (p.H > 1 && (s[1] * es) % 16 != 0) return false;
     if (p.M > 1 && (s[2] * es) % 16 != 0) return false;
-    // whole 16-byte chunks only: a copy never reads past the end of a row
-    if (((int64_t)p.N * es) % 16 != 0) return false;
+    // A copy fetches whole 16-byte chunks: either the rows are whole chunks, or the row stride leaves
+    // room for the last one (a padded row pitch, or a column slice of a wider tensor), so that the
+    // bytes behind the last key of a row are readable; the kernels mask what they read there and write
+    // a partial chunk of dbias element by element.
+    const int64_t row_bytes = (int64_t)p.N * es, padded = (row_bytes + 15) & ~(int64_t)15;
+    if (row_bytes != padded && !(p.M > 1 && s[2] * es >= padded)) return false;
     // one (batch, head) slice is addressed through a 32-bit buffer descriptor
-    if (s[2] < 0 || ((int64_t)(p.M - 1) * s[2] + p.N) * es >= (1ll << 31)) return false;
+    if (s[2] < 0 || (int64_t)(p.M - 1) * s[2] * es + padded >= (1ll << 31)) return false;
     return true;
 }
 
@@ -154,8 +158,8 @@ void note_slow_bias(const char* what, const void* ptr, const int64_t s[4], const
     if (!std::getenv("FA_MI355_VERBOSE") || said.exchange(true)) return;
     std::fprintf(stderr,
                  "libfa_mi355: %s takes the element-wise path (pointer %p, strides %lld/%lld/%lld/%lld elements, N = %d): "
-                 "needs unit key stride, 16-byte aligned base and B/H/M strides, rows of whole 16-byte chunks and "
-                 "(batch, head) slices below 2 GiB\n",
+                 "needs unit key stride, 16-byte aligned base and B/H/M strides, rows of whole 16-byte chunks (or a "
+                 "row stride that covers the last chunk) and (batch, head) slices below 2 GiB\n",
                  what, ptr, (long long)s[0], (long long)s[1], (long long)s[2], (long long)s[3], p.N);
 }
 

@@ -661,13 +661,21 @@ __global__ __launch_bounds__((BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>::NT)
     // per-element path for bias rows that cannot be copied in aligned 16-byte chunks
     auto load_bias_scalar = [&](int mb, unsigned char* dst) {
         if constexpr (TB != 0) {
+            // all loads of a 32-row sub-block in flight together (clamped addresses instead of
+            // branches; what lies outside the bias is masked where it is used)
             const int m0 = mb * BMI;
+            const int nn = my_n < N ? my_n : N - 1;
 #pragma unroll 1
-            for (int row = g; row < BMI; row += 2) {
-                const int m = m0 + row;
-                E val = (E)0.f;
-                if (m < M && my_n < N) val = bp[(int64_t)m * p.sbias.m + (int64_t)my_n * p.sbias.n];
-                reinterpret_cast<E*>(dst)[row * 32 + r] = val;
+            for (int sb = 0; sb < NSUB; sb++) {
+                E vals[16];
+#pragma unroll
+                for (int j = 0; j < 16; j++) {
+                    int m = m0 + sb * 32 + 2 * j + g;
+                    m = m < M ? m : M - 1;
+                    vals[j] = bp[(int64_t)m * p.sbias.m + (int64_t)nn * p.sbias.n];
+                }
+#pragma unroll
+                for (int j = 0; j < 16; j++) reinterpret_cast<E*>(dst)[(sb * 32 + 2 * j + g) * 32 + r] = vals[j];
             }
         }
     };

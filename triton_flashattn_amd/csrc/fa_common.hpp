@@ -461,14 +461,37 @@ template <typename T, int D, int BIAS, bool WITH_V = true> struct KeyStream {
         wait_vmcnt<(BV ? C::BCH : 0) + OPS*(C::LA - 1)>();
         lds_barrier();
         if constexpr (C::ES != 0 && !BV) {
-            // unaligned bias rows or non-unit key stride: one element per lane per row
-            if (lane < 32) {
+            // unaligned bias rows or non-unit key stride: one element per lane, 16 rows per lane,
+            // RB loads in flight together (clamped addresses instead of branches; what lies outside
+            // the bias is masked where it is used)
+            if constexpr (D >= 128 && C::ES == 4) {
+                // (no register to spare in this variant: one row at a time)
+                if (lane < 32) {
 #pragma unroll 1
-                for (int row = 0; row < 32; row++) {
-                    const int n = k * C::BK + lane;
-                    E val = (E)0.f;
-                    if (mw + row < M && n < N) val = bp[(int64_t)(mw + row) * sbm + (int64_t)n * sbn];
-                    *reinterpret_cast<E*>(b_lds(k) + b_off(row, lane)) = val;
+                    for (int row = 0; row < 32; row++) {
+                        const int n = k * C::BK + lane;
+                        E val = (E)0.f;
+                        if (mw + row < M && n < N) val = bp[(int64_t)(mw + row) * sbm + (int64_t)n * sbn];
+                        *reinterpret_cast<E*>(b_lds(k) + b_off(row, lane)) = val;
+                    }
+                }
+            } else {
+                constexpr int RB = D >= 128 ? 4 : 16;  // as many as the registers of the kernel allow
+                const int key = lane & 31;
+                int n = k * C::BK + key;
+                n = n < N ? n : N - 1;
+#pragma unroll 1
+                for (int j0 = 0; j0 < 16; j0 += RB) {
+                    E vals[RB];
+#pragma unroll
+                    for (int j = 0; j < RB; j++) {
+                        int m = mw + 2 * (j0 + j) + (lane >> 5);
+                        m = m < M ? m : M - 1;
+                        vals[j] = bp[(int64_t)m * sbm + (int64_t)n * sbn];
+                    }
+#pragma unroll
+                    for (int j = 0; j < RB; j++)
+                        *reinterpret_cast<E*>(b_lds(k) + b_off(2 * (j0 + j) + (lane >> 5), key)) = vals[j];
                 }
             }
         }

@@ -256,6 +256,40 @@ def _check_bias(bias, q, k):
     return b4
 
 
+def _bias_rows_ok(b):
+    """Whether the kernels can fetch the rows of a 4-D bias in aligned 16-byte chunks (the rule of the
+    C ABI): unit key stride, aligned base and strides, and rows that are whole chunks or whose stride
+    covers their last chunk.  A bias without a row dimension is read once per work-group, any layout."""
+    es, N = b.element_size(), b.shape[3]
+    if b.shape[2] == 1 or b.stride(2) == 0:
+        return True
+    if (N > 1 and b.stride(3) != 1) or b.data_ptr() % 16 != 0:
+        return False
+    if any(b.shape[i] > 1 and (b.stride(i) * es) % 16 != 0 for i in range(3)):
+        return False
+    padded = -(-N * es // 16) * 16
+    return N * es == padded or b.stride(2) * es >= padded
+
+
+def _empty_padded_rows(shape, dtype, device):
+    """An uninitialised tensor of `shape` whose rows start at multiples of 16 bytes and own the rest
+    of their last 16-byte chunk (a view of an allocation with a padded last dimension)."""
+    per = 16 // torch.empty((), dtype=dtype).element_size()
+    n_pad = -(-shape[-1] // per) * per
+    return torch.empty(tuple(shape[:-1]) + (n_pad,), dtype=dtype, device=device)[..., :shape[-1]]
+
+
+def _bias_kernel_layout(b):
+    """b, or a copy with padded rows when the kernels would have to read b element by element (an odd
+    number of keys, a misaligned view): one pass over the bias instead of a several times slower
+    forward and backward."""
+    if _bias_rows_ok(b):
+        return b
+    out = _empty_padded_rows(b.shape, b.dtype, b.device)
+    out.copy_(b)
+    return out
+
+
 def _check_causal(causal, M, N):
     if causal and M != N:
         raise ValueError("causal attention needs as many queries as keys, got M=%d, N=%d" % (M, N))
@@ -328,11 +362,11 @@ def _bias_grad_like(bias, B, H, M, N):
     computed densely and summed here (an (M, N) accumulator per output slice does not fit the
     kernels)."""
     full = (B, H, M, N)
-    if tuple(bias.shape) == full or (bias.shape[2] == 1 and (bias.shape[3] == N)):
-        dbias = torch.empty(bias.shape, dtype=bias.dtype, device=bias.device)
-        return dbias, (lambda t: t)
-    dense = torch.empty(full, dtype=bias.dtype, device=bias.device)
-    return dense, (lambda t: t.sum_to_size(bias.shape))
+    if bias.shape[2] == 1 and bias.shape[3] == N:
+        return torch.empty(bias.shape, dtype=bias.dtype, device=bias.device), (lambda t: t)
+    if tuple(bias.shape) == full:
+        return _empty_padded_rows(full, bias.dtype, bias.device), (lambda t: t)
+    return _empty_padded_rows(full, bias.dtype, bias.device), (lambda t: t.sum_to_size(bias.shape))
 
 
 # --------------------------------------------------------------------------------------------
@@ -360,6 +394,8 @@ class FlashAttentionFn(torch.autograd.Function):
                 raise ValueError("give either a bias tensor or ALiBi slopes, not both")
             bias = AlibiBias(alibi_slopes)
         bias = _check_bias(bias, q, k)
+        if isinstance(bias, torch.Tensor):
+            bias = _bias_kernel_layout(bias)
         _check_causal(causal, q.shape[1], k.shape[1])
         sm_scale = (q.shape[-1] ** -0.5) if sm_scale is None else sm_scale
         is_bias = bias is not None
@@ -434,6 +470,8 @@ class FlashAttentionQKVPackedFn(torch.autograd.Function):
                 raise ValueError("give either a bias tensor or ALiBi slopes, not both")
             bias = AlibiBias(alibi_slopes)
         bias = _check_bias(bias, q, k)
+        if isinstance(bias, torch.Tensor):
+            bias = _bias_kernel_layout(bias)
         sm_scale = (qkv.shape[-1] ** -0.5) if sm_scale is None else sm_scale
         is_bias = bias is not None
         alibi = isinstance(bias, AlibiBias)
@@ -519,6 +557,8 @@ def _op_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, bias: Optional[to
     if v.shape[-1] != q.shape[-1]:
         raise ValueError("flash_attention_op needs v with the head dim of q")
     bias = _check_bias(bias, q, k)
+    if bias is not None:
+        bias = _bias_kernel_layout(bias)
     _check_causal(causal, q.shape[1], k.shape[1])
     return _flash_attn_fwd(q, k, v, bias, causal, sm_scale)
 
@@ -537,11 +577,13 @@ def _op_bwd(do: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     dbias, finish = None, None
     b4 = _check_bias(bias, q, k)
+    if b4 is not None:
+        b4 = _bias_kernel_layout(b4)
     if bias_grad:
         dbias, finish = _bias_grad_like(b4, B, H, M, k.shape[1])
     _flash_attn_bwd(do, q, k, v, o, b4, causal, sm_scale, lse, dq, dk, dv, dbias)
     # an operator cannot return None: no bias gradient is an empty tensor
-    return dq, dk, dv, (finish(dbias).reshape(bias.shape) if bias_grad else q.new_empty((0,)))
+    return dq, dk, dv, (finish(dbias).reshape(bias.shape).contiguous() if bias_grad else q.new_empty((0,)))
 
 
 @_op_bwd.register_fake

@@ -205,6 +205,29 @@ def test_v_with_another_head_dim(gpu_device):
         check(ours, run_oracle(q, k, v, do, bias, causal), "Dqk%d Dv%d" % (d_qk, d_v))
 
 
+@pytest.mark.parametrize("D", [8, 40, 80, 96, 160, 192])
+def test_head_dims_the_kernels_are_not_built_for(gpu_device, D):
+    """Head dims between those of the kernels run zero-padded to the next one; sm_scale keeps its
+    default of the true head dim (flash_attention.py:789)."""
+    B, M, N, H = 2, 150, 170, 2
+    for i, (kind, causal) in enumerate([(None, True), ("bf16", False), ("bool", False)]):
+        n = M if causal else N
+        q, k, v, do, bias = make_inputs(gpu_device, B, M, n, H, D, torch.bfloat16, kind, seed=3 * D + i)
+        ours = run_ours(q, k, v, do, bias, causal)
+        assert ours["out"].shape == q.shape and ours["dk"].shape == k.shape and ours["dv"].shape == v.shape
+        check(ours, run_oracle(q, k, v, do, bias, causal), "D%d %s causal=%s" % (D, kind, causal))
+    # packed
+    g = torch.Generator().manual_seed(D)
+    qkv = torch.randn(B, M, 3, H, D, generator=g).bfloat16().to(gpu_device).requires_grad_(True)
+    do = torch.randn(B, M, H, D, generator=g).bfloat16().to(gpu_device)
+    out = flash_attention_qkvpacked_fn(qkv, None, True)
+    out.backward(do)
+    ref = run_oracle(qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], do, None, True)
+    assert qkv.grad.shape == qkv.shape
+    check({"out": out.detach(), "dq": qkv.grad[:, :, 0], "dk": qkv.grad[:, :, 1], "dv": qkv.grad[:, :, 2], "dbias": None},
+          ref, "packed D%d" % D)
+
+
 def test_gradients_nobody_asks_for_are_skipped(gpu_device):
     """Only the kernels whose outputs are wanted run, and what they write equals the full run."""
     B, M, N, H, D = 2, 300, 260, 2, 64

@@ -79,13 +79,14 @@ def test_rejects_bad_arguments(oracle_backend):
         flash_attention_fn(q.float(), k.float(), v.float())              # dtype
     with pytest.raises(TypeError):
         flash_attention_fn(q, k.half(), v)                               # mixed dtype
+    q300, k300, v300 = _qkv(D=300)
     with pytest.raises(ValueError):
-        flash_attention_fn(q[..., :8], k[..., :8], v[..., :8])           # head dim 8 (flash_attention.py:776)
+        flash_attention_fn(q300, k300, v300)                             # head dim above 256 (flash_attention.py:776)
     with pytest.raises(ValueError):
         flash_attention_fn(q, k[..., :8].repeat(1, 1, 1, 4), v)         # k head dim != q head dim (:775)
     q32, k32, v32 = _qkv(D=32)
     with pytest.raises(ValueError):
-        flash_attention_fn(q32, k32, v32[..., :8])                       # v head dim 8
+        flash_attention_fn(q32, k32, v300)                               # v head dim above 256
     with pytest.raises(ValueError):
         flash_attention_fn(q, k[:, :, :1], v[:, :, :1])                  # head count
     with pytest.raises(ValueError):
@@ -232,7 +233,8 @@ def test_alibi_bias_matches_materialized(oracle_backend):
 def test_v_with_another_head_dim(oracle_backend):
     g = torch.Generator().manual_seed(5)
     B, M, N, H = 2, 6, 9, 2
-    for d_qk, d_v in ((16, 32), (64, 16)):
+    # ... and head dims between those of the kernels (zero-padded to the next one)
+    for d_qk, d_v in ((16, 32), (64, 16), (8, 8), (80, 80), (40, 96)):
         q = torch.randn(B, M, H, d_qk, generator=g).bfloat16().requires_grad_(True)
         k = torch.randn(B, N, H, d_qk, generator=g).bfloat16().requires_grad_(True)
         v = torch.randn(B, N, H, d_v, generator=g).bfloat16().requires_grad_(True)
@@ -245,6 +247,9 @@ def test_v_with_another_head_dim(oracle_backend):
         for name, t in (("dq", q), ("dk", k), ("dv", v)):
             assert t.grad.shape == t.shape
             assert torch.allclose(t.grad.float(), ref[name], atol=3e-2, rtol=3e-2), (name, d_qk, d_v)
+    qkv = torch.randn(1, 8, 3, H, 24, generator=g).bfloat16().requires_grad_(True)   # packed, head dim 24
+    flash_attention_qkvpacked_fn(qkv, None, True).sum().backward()
+    assert qkv.grad.shape == qkv.shape and torch.isfinite(qkv.grad.float()).all()
 
 
 def test_gradients_nobody_asks_for_are_not_computed(oracle_backend):

@@ -201,7 +201,13 @@ def _as_kernel_layout(t):
     return t if _kernel_layout_ok(t) else t.contiguous()
 
 
-def _check_qkv(q, k, v):
+def _kernel_head_dim(d):
+    """The head dim the kernels run a head dim of d at (the next one they are built for)."""
+    return next(x for x in _HEAD_DIMS if x >= d)
+
+
+def _check_qkv(q, k, v, any_head_dim=False):
+    """any_head_dim: the caller zero-pads head dims the kernels are not built for (1 .. 256)."""
     for name, t in (("q", q), ("k", k), ("v", v)):
         if not isinstance(t, torch.Tensor):
             raise TypeError("%s must be a torch.Tensor" % name)
@@ -212,12 +218,13 @@ def _check_qkv(q, k, v):
     if k.dtype != q.dtype or v.dtype != q.dtype:
         raise TypeError("q, k, v must share one dtype, got %s, %s, %s" % (q.dtype, k.dtype, v.dtype))
     B, M, H, D = q.shape
-    if D not in _HEAD_DIMS:
-        raise ValueError("head dim must be one of %s, got %d" % (_HEAD_DIMS, D))
+    for name, d in (("head dim", D), ("v head dim", v.shape[-1])):
+        if any_head_dim and not 1 <= d <= _HEAD_DIMS[-1]:
+            raise ValueError("%s must be between 1 and %d, got %d" % (name, _HEAD_DIMS[-1], d))
+        if not any_head_dim and d not in _HEAD_DIMS:
+            raise ValueError("%s must be one of %s, got %d" % (name, _HEAD_DIMS, d))
     if k.shape[-1] != D:
         raise ValueError("k head dim %d differs from q head dim %d" % (k.shape[-1], D))
-    if v.shape[-1] not in _HEAD_DIMS:
-        raise ValueError("v head dim must be one of %s, got %d" % (_HEAD_DIMS, v.shape[-1]))
     N = k.shape[1]
     if k.shape[0] != B or v.shape[0] != B or k.shape[2] != H or v.shape[2] != H or v.shape[1] != N:
         raise ValueError("inconsistent shapes: q %s, k %s, v %s" % (tuple(q.shape), tuple(k.shape), tuple(v.shape)))
@@ -388,7 +395,7 @@ class FlashAttentionFn(torch.autograd.Function):
     @staticmethod
     @_fwd_amp
     def forward(ctx, q, k, v, bias=None, causal=False, sm_scale=None, alibi_slopes=None):
-        _check_qkv(q, k, v)
+        _check_qkv(q, k, v, any_head_dim=True)
         if alibi_slopes is not None:
             if bias is not None:
                 raise ValueError("give either a bias tensor or ALiBi slopes, not both")
@@ -404,10 +411,11 @@ class FlashAttentionFn(torch.autograd.Function):
         if is_bias_trainable and not alibi and bias.dtype == torch.bool:
             raise TypeError("a bool bias cannot require grad")
 
-        # v with another head dim than q and k: the narrower side is zero-padded (zeros add nothing
-        # to a score, and the padded columns of the output are dropped)
+        # v with another head dim than q and k, or a head dim the kernels are not built for (80, 96,
+        # ...): zero-padded to the next one they are (zeros add nothing to a score, and the padded
+        # columns of the output are dropped)
         d_qk, d_v = q.shape[-1], v.shape[-1]
-        D = max(d_qk, d_v)
+        D = _kernel_head_dim(max(d_qk, d_v))
         qp, kp, vp = _pad_head_dim(q, D), _pad_head_dim(k, D), _pad_head_dim(v, D)
 
         o, lse = _flash_attn_fwd(qp, kp, vp, bias, causal, sm_scale)
@@ -543,6 +551,9 @@ def flash_attention_qkvpacked_fn(qkv, bias=None, causal=False, sm_scale=None):
     """Self-attention on a packed qkv (B, seqlen, 3, H, D); bias as for flash_attention_fn with
     M = N = seqlen.  The gradient comes back packed in one tensor.  Returns out (B, seqlen, H, D)."""
     (qkv,) = _autocast_inputs(qkv)
+    if isinstance(qkv, torch.Tensor) and qkv.dim() == 5 and qkv.shape[2] == 3 and qkv.shape[-1] not in _HEAD_DIMS:
+        # a head dim that needs padding: the packed layout is lost anyway
+        return flash_attention_fn(qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], bias, causal, sm_scale)
     bias, slopes = _split_bias(bias)
     return FlashAttentionQKVPackedFn.apply(qkv, bias, causal, sm_scale, slopes)
 

@@ -6,7 +6,7 @@ import torch
 
 import triton_flashattn_amd.flash_attention as fa_mod
 from triton_flashattn_amd import _native
-from triton_flashattn_amd.flash_attention import _flash_attn_fwd
+from triton_flashattn_amd.flash_attention import _flash_attn_fwd, flash_attention_fn
 from oracle.attention_oracle import LN2, attention_forward, attention_forward_streamed
 from test_gpu_parity import GRAD_RTOL, OUT_ATOL, check, make_inputs, rel_l2, run_oracle, run_ours
 
@@ -220,3 +220,54 @@ def test_bias_rows_that_are_not_whole_chunks(gpu_device, D, kind):
         check(res, ref, "slice %s D%d case %d" % (kind, D, i))
         if trainable:
             assert (dwide[..., N:] == 7.0).all(), "the columns behind the dbias slice were written"
+
+
+# ---------------------------------------------------------------- a (batch, head) slice of the bias of 2 GiB
+def test_bias_slice_of_two_gib_equals_its_halves(gpu_device):
+    """M = N = 32768 with a bf16 bias: one (batch, head) slice is 2 GiB, beyond the 32-bit offsets of
+    the copy path, so bias and dBias go element by element with 64-bit indices.  Too large for the CPU
+    oracle; attention decomposes over blocks of query rows, and each half of the rows (a 1 GiB slice
+    on the copy path, which the smaller tests pin to the oracle) must give the same rows of out, dq
+    and dBias, and dk, dv that add up."""
+    B, H, S, D = 1, 1, 32768, 16
+    g = torch.Generator(device=gpu_device).manual_seed(9)
+    mk = lambda *s: torch.randn(*s, device=gpu_device, generator=g).bfloat16()
+    q, k, v, do = mk(B, S, H, D), mk(B, S, H, D), mk(B, S, H, D), mk(B, S, H, D)
+    bias = mk(B, H, S, S)
+    assert bias[0, 0].numel() * bias.element_size() == 1 << 31
+    full = run_ours(q, k, v, do, bias.requires_grad_(True), False)
+    half = S // 2
+    dk_sum, dv_sum = torch.zeros_like(k, dtype=torch.float32), torch.zeros_like(v, dtype=torch.float32)
+    for lo in (0, half):
+        rows = slice(lo, lo + half)
+        part = run_ours(q[:, rows], k, v, do[:, rows], bias.detach()[:, :, rows].requires_grad_(True), False)
+        assert (part["out"].float() - full["out"][:, rows].float()).abs().max().item() <= 1e-2
+        assert rel_l2(part["dq"], full["dq"][:, rows].float()) <= 1e-2
+        assert rel_l2(part["dbias"], full["dbias"][:, :, rows].float()) <= 1e-2
+        dk_sum += part["dk"].float()
+        dv_sum += part["dv"].float()
+    assert rel_l2(full["dk"], dk_sum) <= 2e-2 and rel_l2(full["dv"], dv_sum) <= 2e-2
+
+
+def test_long_sequences_decompose(gpu_device):
+    """65536 keys, beyond what the CPU oracle finishes in seconds: the causal result on a prefix of
+    the sequence is the result of the prefix alone, and the rows of a non-causal call are those of a
+    call on half of the queries."""
+    B, H, S, D = 1, 2, 65536, 64
+    g = torch.Generator(device=gpu_device).manual_seed(10)
+    mk = lambda *s: (torch.randn(*s, device=gpu_device, generator=g) * 0.5).half()
+    q, k, v, do = mk(B, S, H, D), mk(B, S, H, D), mk(B, S, H, D), mk(B, S, H, D)
+    half = S // 2
+    # causal: rows below `half` see keys below `half` only
+    full = flash_attention_fn(q, k, v, None, True)
+    pre = flash_attention_fn(q[:, :half], k[:, :half], v[:, :half], None, True)
+    assert torch.equal(full[:, :half], pre)
+    # non-causal, with gradients: the second half of the queries
+    full = run_ours(q, k, v, do, None, False)
+    rows = slice(half, S)
+    part = run_ours(q[:, rows], k, v, do[:, rows], None, False)
+    assert torch.equal(part["out"], full["out"][:, rows])
+    assert rel_l2(part["dq"], full["dq"][:, rows].float()) <= 1e-3
+    other = run_ours(q[:, :half], k, v, do[:, :half], None, False)
+    assert rel_l2(full["dk"], part["dk"].float() + other["dk"].float()) <= 2e-2
+    assert rel_l2(full["dv"], part["dv"].float() + other["dv"].float()) <= 2e-2

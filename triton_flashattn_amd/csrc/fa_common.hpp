@@ -353,9 +353,18 @@ template <typename T, int D, int BIAS, bool WITH_V = true> struct KeyStream {
     const E* bp;              // (batch, head) slices
     int64_t sk, sv, sbm, sbn; // row strides of K and V, row and key stride of the bias (elements)
     int M, N, mw, lane;
-    unsigned k_off[C::KD], v_off[C::KD];
-    int c_idx[C::KD];
+    // LEAN (rows of 32 chunks, head dim 256): the per-lane offsets of the KD copies are formed from
+    // three per-lane constants when a copy is issued, instead of being held in 3 KD registers that
+    // such a kernel does not have: a copy of chunk c = 64 ci + l reads row 2 ci + g (g = l / 32), chunk
+    // (l % 32) ^ f(2 ci + g), and f(2 ci + g) = (g << 2) ^ F(ci) with F the same for every lane.
+    static constexpr bool LEAN = C::CPR == 32;
+    unsigned k_off[LEAN ? 1 : C::KD], v_off[LEAN ? 1 : C::KD];
+    int c_idx[LEAN ? 1 : C::KD];
+    unsigned lean_x16, lean_rk, lean_rv;  // ((l % 32) ^ (g << 2)) * 16, byte offsets of row g of K and of V
+    int wave_s;                           // wave index (scalar)
     unsigned lds_kv, lds_bias;  // LDS addresses (scalar) of the K slots and of this wave's bias ring
+    // chunk index of copy i of this wave (scalar)
+    __device__ __forceinline__ int copy_idx(int i) const { return LEAN ? (wave_s * C::KD + i) % C::NKD : c_idx[i]; }
 
     // K / V rows of a step: NKD copies of 1 KB each; copy ci fills bytes [1024 ci, 1024 ci + 1024) of
     // the swizzled slot, so lane l of it fetches the chunk that lives at slot position 64 ci + l
@@ -369,13 +378,21 @@ template <typename T, int D, int BIAS, bool WITH_V = true> struct KeyStream {
         bias_lds = smem + C::KV_BYTES + wave * C::NBS * C::BSLOT;
         lds_kv = lds_addr_of(smem);
         lds_bias = lds_kv + C::KV_BYTES + wave * C::NBS * C::BSLOT;
+        wave_s = wave;
+        if constexpr (LEAN) {
+            const int g = lane >> 5;
+            lean_x16 = (unsigned)(((lane & 31) ^ (g << 2)) << 4);
+            lean_rk = (unsigned)(g * (int)sk * 2);
+            lean_rv = (unsigned)(g * (int)sv * 2);
+        } else {
 #pragma unroll
-        for (int i = 0; i < C::KD; i++) {
-            c_idx[i] = (wave * C::KD + i) % C::NKD;
-            const int c = c_idx[i] * 64 + lane;
-            const int row = c / C::CPR, src = (c % C::CPR) ^ SW::f(row);
-            k_off[i] = (unsigned)(row * (int)sk * 2 + src * 16);
-            v_off[i] = (unsigned)(row * (int)sv * 2 + src * 16);
+            for (int i = 0; i < C::KD; i++) {
+                c_idx[i] = (wave * C::KD + i) % C::NKD;
+                const int c = c_idx[i] * 64 + lane;
+                const int row = c / C::CPR, src = (c % C::CPR) ^ SW::f(row);
+                k_off[i] = (unsigned)(row * (int)sk * 2 + src * 16);
+                v_off[i] = (unsigned)(row * (int)sv * 2 + src * 16);
+            }
         }
     }
     __device__ __forceinline__ const T* k_lds(int k) const { return reinterpret_cast<const T*>(smem + (k % C::NKV) * C::STEP_BYTES); }
@@ -401,17 +418,27 @@ template <typename T, int D, int BIAS, bool WITH_V = true> struct KeyStream {
         const bool full = n0 + C::BK <= N;
 #pragma unroll
         for (int i = 0; i < C::KD; i++) {
-            unsigned ko = k_off[i], vo = v_off[i];
+            const int ci = copy_idx(i);
+            unsigned ko, vo;
+            if constexpr (LEAN) {
+                const int r0 = 2 * ci;  // first of the two rows of this copy
+                const unsigned x = lean_x16 ^ (unsigned)((((r0 & 3) << 2) | ((r0 >> 2) & 3)) << 4);
+                ko = x + lean_rk + (unsigned)(r0 * (int)sk * 2);
+                vo = x + lean_rv + (unsigned)(r0 * (int)sv * 2);
+            } else {
+                ko = k_off[i];
+                vo = v_off[i];
+            }
             if (!full) {
-                const int c = c_idx[i] * 64 + lane;
+                const int c = ci * 64 + lane;
                 int row = c / C::CPR;
                 const int src = (c % C::CPR) ^ SW::f(row);
                 row = row < N - n0 ? row : N - 1 - n0;
                 ko = (unsigned)(row * (int)sk * 2 + src * 16);
                 vo = (unsigned)(row * (int)sv * 2 + src * 16);
             }
-            lds_copy16(kt, ko, k_dst + c_idx[i] * 1024);
-            if constexpr (WITH_V) lds_copy16(vt, vo, v_dst + c_idx[i] * 1024);
+            lds_copy16(kt, ko, k_dst + ci * 1024);
+            if constexpr (WITH_V) lds_copy16(vt, vo, v_dst + ci * 1024);
         }
     }
     // Bias slice of this wave for step k (32 rows x 32 keys) -> ring slot k % NBS.  Position c =

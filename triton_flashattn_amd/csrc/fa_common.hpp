@@ -353,10 +353,13 @@ template <typename T, int D, int BIAS, bool WITH_V = true> struct KeyStream {
     const E* bp;              // (batch, head) slices
     int64_t sk, sv, sbm, sbn; // row strides of K and V, row and key stride of the bias (elements)
     int M, N, mw, lane;
-    // LEAN (rows of 32 chunks, head dim 256): the per-lane offsets of the KD copies are formed from
-    // three per-lane constants when a copy is issued, instead of being held in 3 KD registers that
-    // such a kernel does not have: a copy of chunk c = 64 ci + l reads row 2 ci + g (g = l / 32), chunk
-    // (l % 32) ^ f(2 ci + g), and f(2 ci + g) = (g << 2) ^ F(ci) with F the same for every lane.
+    // LEAN (rows of LEAN_CPR chunks): the per-lane offsets of the KD copies are formed from three
+    // per-lane constants when a copy is issued, instead of being held in 3 KD registers that such a
+    // kernel does not have: a copy of chunk c = 64 ci + l reads row r0 + q (r0 = (64 / CPR) ci, q =
+    // l / CPR), chunk (l % CPR) ^ f(r0 + q), and f(r0 + q) = (q << 2) ^ f(r0) with f(r0) the same for
+    // every lane (holds for rows of 16 and of 32 chunks).
+    // Used at head dim 256; at 128 the kernels have the registers and the extra address arithmetic per
+    // copy buys nothing.
     static constexpr bool LEAN = C::CPR == 32;
     unsigned k_off[LEAN ? 1 : C::KD], v_off[LEAN ? 1 : C::KD];
     int c_idx[LEAN ? 1 : C::KD];
@@ -380,10 +383,11 @@ template <typename T, int D, int BIAS, bool WITH_V = true> struct KeyStream {
         lds_bias = lds_kv + C::KV_BYTES + wave * C::NBS * C::BSLOT;
         wave_s = wave;
         if constexpr (LEAN) {
-            const int g = lane >> 5;
-            lean_x16 = (unsigned)(((lane & 31) ^ (g << 2)) << 4);
-            lean_rk = (unsigned)(g * (int)sk * 2);
-            lean_rv = (unsigned)(g * (int)sv * 2);
+            static_assert(C::CPR == 16 || C::CPR == 32, "rows of 16 or 32 chunks");
+            const int q = lane / C::CPR;
+            lean_x16 = (unsigned)(((lane % C::CPR) ^ (q << 2)) << 4);
+            lean_rk = (unsigned)(q * (int)sk * 2);
+            lean_rv = (unsigned)(q * (int)sv * 2);
         } else {
 #pragma unroll
             for (int i = 0; i < C::KD; i++) {
@@ -421,7 +425,7 @@ template <typename T, int D, int BIAS, bool WITH_V = true> struct KeyStream {
             const int ci = copy_idx(i);
             unsigned ko, vo;
             if constexpr (LEAN) {
-                const int r0 = 2 * ci;  // first of the two rows of this copy
+                const int r0 = (64 / C::CPR) * ci;  // first of the rows of this copy
                 const unsigned x = lean_x16 ^ (unsigned)((((r0 & 3) << 2) | ((r0 >> 2) & 3)) << 4);
                 ko = x + lean_rk + (unsigned)(r0 * (int)sk * 2);
                 vo = x + lean_rv + (unsigned)(r0 * (int)sv * 2);

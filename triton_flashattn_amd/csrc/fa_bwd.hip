@@ -438,13 +438,16 @@ template <int D, int BIAS, bool OCC2 = false> struct BwdCfg {
     // a copy has LA - 1 whole steps and the rest of its own to land before the barrier that
     // publishes it.
     static constexpr int DS_BYTES = (BIAS == 2 || BIAS == 3) ? BN * DSS * 2 : 0;  // dS^T tiles (dBias)
+    // The LSE (delta) values of a block: a copy is 64 lanes wide, so a slot is 64 floats; with 32-row
+    // blocks the upper lanes copy the same 32 values again (no lane mask, no branch around the copy).
+    static constexpr int STAT_BYTES = 64 * 4;
     static constexpr int P_BYTES = 4 * NSUB * 64 * 16 * WPR;  // P hand-off: 16 floats per lane per sub-block
     static constexpr int BT_BYTES = BMI * 32 * ES;         // bias slice of one S-wave
     // LDS bytes with copies la blocks ahead: la + 1 dO buffers and bias slots, la + 2 Q buffers and
     // one more if the dK product of a block is deferred by a step (so that it does not wait for
     // the dS of the same step)
     static constexpr int lds_total(int la, int defer) {
-        return (2 * la + 3 + defer) * (Q_BYTES + BMI * 4) + DS_BYTES + 2 * P_BYTES + WPR * (la + 1) * BT_BYTES;
+        return (2 * la + 3 + defer) * (Q_BYTES + STAT_BYTES) + DS_BYTES + 2 * P_BYTES + WPR * (la + 1) * BT_BYTES;
     }
     static constexpr int LA = D > 128 ? 1 : (lds_total(3, 1) <= LDS_LIMIT ? 3 : 2);
     static constexpr bool DEFER_DK = D <= 128 && lds_total(LA, 1) <= LDS_LIMIT;
@@ -455,8 +458,8 @@ template <int D, int BIAS, bool OCC2 = false> struct BwdCfg {
     static constexpr int OFF_DS = OFF_DO + NDOB * Q_BYTES;
     static constexpr int OFF_P = OFF_DS + DS_BYTES;        // two hand-off buffers
     static constexpr int OFF_LSE = OFF_P + 2 * P_BYTES;
-    static constexpr int OFF_DELTA = OFF_LSE + NQB * BMI * 4;
-    static constexpr int OFF_BIAS = OFF_DELTA + NDOB * BMI * 4;
+    static constexpr int OFF_DELTA = OFF_LSE + NQB * STAT_BYTES;
+    static constexpr int OFF_BIAS = OFF_DELTA + NDOB * STAT_BYTES;
     static constexpr int LOOP_BYTES = OFF_BIAS + WPR * RING * BT_BYTES;
     static constexpr int LDS_BYTES = LOOP_BYTES;
     static_assert(LDS_BYTES <= LDS_LIMIT, "LDS budget of the configuration");
@@ -607,7 +610,11 @@ __global__ __launch_bounds__((BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>::NT)
         for (int i = 0; i < C::QD; i++) {
             unsigned o = off[i];
             if (!full) {
-                const int c = c_idx[i] * 64 + lane;
+                // (rare: the lane index passes through an empty asm so that these per-lane values are
+                // formed here and not kept in registers across the loops)
+                int lane_here = lane;
+                asm volatile("" : "+v"(lane_here));
+                const int c = c_idx[i] * 64 + lane_here;
                 int row = c / CPR;
                 const int src = (c % CPR) ^ SW::f(row);
                 row = row < M - m0 ? row : M - 1 - m0;
@@ -618,11 +625,9 @@ __global__ __launch_bounds__((BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>::NT)
     };
     // one float per row
     auto issue_stat = [&](const float* src, int mb, unsigned dst) {
-        if (lane < BMI) {
-            int m = mb * BMI + lane;
-            m = m < M ? m : M - 1;
-            lds_copy4(uniform_ptr(src), (unsigned)m * 4u, dst);
-        }
+        int m = mb * BMI + lane % BMI;
+        m = m < M ? m : M - 1;
+        lds_copy4(uniform_ptr(src), (unsigned)m * 4u, dst);
     };
     // bias slice (BMI rows x 32 keys) of query block mb -> ring slot.  Chunk c = 64 it + lane of the
     // slice (row c / BCPR, 16-byte chunk c % BCPR) lands at byte 16 c of the slot, i.e. the slot
@@ -648,16 +653,67 @@ __global__ __launch_bounds__((BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>::NT)
     // all four waves of a role copy the 32 or 64 floats, which keeps their counts alike
     auto issue_q = [&](int mb) {
         issue_rows(qp, p.sq.s, cq_off, mb, lds_base + (mb % C::NQB) * C::Q_BYTES);
-        issue_stat(lsep, mb, lds_base + C::OFF_LSE + (mb % C::NQB) * BMI * 4);
+        issue_stat(lsep, mb, lds_base + C::OFF_LSE + (mb % C::NQB) * C::STAT_BYTES);
     };
     auto issue_do = [&](int mb) {
         issue_rows(dop, p.sdo.s, cdo_off, mb, lds_base + C::OFF_DO + (mb % C::NDOB) * C::Q_BYTES);
-        issue_stat(deltap, mb, lds_base + C::OFF_DELTA + (mb % C::NDOB) * BMI * 4);
+        issue_stat(deltap, mb, lds_base + C::OFF_DELTA + (mb % C::NDOB) * C::STAT_BYTES);
     };
     // Issuing a copy stalls the wave while the memory pipeline of the CU is backed up, so the
     // copies are dealt out between the roles: Q and the bias go with the S-waves, dO with the
     // dP-waves.
     constexpr bool Q_BY_S = true, DO_BY_S = false;
+    static_assert(Q_BY_S && !DO_BY_S, "the running pointers of the interior steps are laid out for this deal");
+    // Interior steps (every block they touch is whole, in range and unmasked: all but the first and
+    // the last few of a tile) walk the query blocks in order, so their copies keep running block
+    // pointers in scalar registers, one 64-bit add per block, and need no clamps; run_start() points
+    // them at the first blocks an interior loop issues.
+    // (The kernels that run two work-groups per CU have 128 registers per wave and no room for the
+    // second copy of the loop: they run every step in its general form.)
+    constexpr bool IN_LOOPS = !bwd_occ2(D, BIAS);
+    const int n_full = M / BMI;  // blocks whose rows all exist
+    uint64_t run_rows = 0, run_stat = 0, run_bias = 0;  // Q and LSE (role that issues Q) or dO and delta; bias slices
+    unsigned bias_off0 = 0;  // this lane's byte offset in the first bias copy of a block, from the block's first row
+    if constexpr (TB != 0) {
+        int nn = nw + (lane % C::BCPR) * C::EPC;
+        nn = nn < N ? nn : 0;
+        bias_off0 = (unsigned)(((int64_t)(lane / C::BCPR) * p.sbias.m + nn) * C::ES);
+    }
+    auto run_start = [&](const T* rows, int64_t row_stride, const float* stat, int mb, int mb_bias) {
+        run_rows = uniform_ptr(rows + (int64_t)mb * BMI * row_stride);
+        run_stat = uniform_ptr(stat + (int64_t)mb * BMI);
+        if constexpr (TB != 0) run_bias = uniform_ptr(bp + (int64_t)mb_bias * BMI * p.sbias.m);
+    };
+    // the next block of Q (or dO) with its LSE (or delta): QD + 1 copies, like issue_q / issue_do
+    // (the caller has passed the running pointers through settle_ptrs() since they were last advanced)
+    auto issue_next_rows = [&](int64_t row_stride, const unsigned (&off)[C::QD], unsigned dst, unsigned stat_dst) {
+#pragma unroll
+        for (int i = 0; i < C::QD; i++) lds_copy16(run_rows, off[i], dst + c_idx[i] * 1024);
+        run_rows += (uint64_t)(BMI * 2) * (uint64_t)row_stride;
+        // (the lane index passes through an empty asm so that the offset is formed here, two
+        // instructions, and does not hold a register across the loop)
+        unsigned lane_here = (unsigned)lane;
+        asm volatile("" : "+v"(lane_here));
+        lds_copy4(run_stat, (lane_here % BMI) * 4u, stat_dst);
+        run_stat += BMI * 4;
+    };
+    auto issue_next_q = [&](int mb) {
+        const unsigned slot = (unsigned)mb % C::NQB;
+        issue_next_rows(p.sq.s, cq_off, lds_base + slot * C::Q_BYTES, lds_base + C::OFF_LSE + slot * C::STAT_BYTES);
+    };
+    auto issue_next_do = [&](int mb) {
+        const unsigned slot = (unsigned)mb % C::NDOB;
+        issue_next_rows(p.sdo.s, cdo_off, lds_base + C::OFF_DO + slot * C::Q_BYTES, lds_base + C::OFF_DELTA + slot * C::STAT_BYTES);
+    };
+    auto issue_next_bias = [&](int mb) {
+        if constexpr (TB != 0) {
+            const unsigned dst = lds_base + C::OFF_BIAS + (kb * C::RING + (unsigned)(mb - mb_first) % C::RING) * C::BT_BYTES;
+            const unsigned rows_step = (unsigned)((64 / C::BCPR) * (int)p.sbias.m * C::ES);  // the rows one copy covers
+#pragma unroll
+            for (int it = 0; it < C::BCH; it++) lds_copy16(run_bias, bias_off0 + it * rows_step, dst + it * 1024);
+            run_bias += (uint64_t)(BMI * C::ES) * (uint64_t)p.sbias.m;
+        }
+    };
     // per-element path for bias rows that cannot be copied in aligned 16-byte chunks
     auto load_bias_scalar = [&](int mb, unsigned char* dst) {
         if constexpr (TB != 0) {
@@ -751,6 +807,9 @@ __global__ __launch_bounds__((BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>::NT)
     // ring slots of a block index that may run one or two blocks below zero at the first steps
     auto q_tile = [&](int mb) { return lds_base + (unsigned)(((mb < 0 ? 0 : mb) % C::NQB) * C::Q_BYTES); };
     auto do_tile = [&](int mb) { return lds_base + (unsigned)(C::OFF_DO + ((mb < 0 ? 0 : mb) % C::NDOB) * C::Q_BYTES); };
+    // the same for the interior steps, whose block indices are never negative
+    auto q_tile_in = [&](int mb) { return lds_base + ((unsigned)mb % C::NQB) * C::Q_BYTES; };
+    auto do_tile_in = [&](int mb) { return lds_base + C::OFF_DO + ((unsigned)mb % C::NDOB) * C::Q_BYTES; };
 
     if (s_wave) {
         // ================================ S-wave ================================
@@ -770,7 +829,9 @@ __global__ __launch_bounds__((BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>::NT)
             load_rows(q_tile(mb_first), a_rows);
             mma_rows(a_rows, sacc);
         }
-        auto s_step = [&](int t) {
+        auto s_step = [&](int t, auto in_tag) {
+            // IN: an interior step: blocks t .. t + 2 + LA are whole and in range, block t + 1 needs no mask
+            constexpr bool IN = decltype(in_tag)::value;
             const int nb = t + 1;  // the block whose P is produced in this step
             T8 op_next[NSUB][2];
             // Copies for the steps to come (their buffers were last read one step ago).  With a bias
@@ -778,13 +839,20 @@ __global__ __launch_bounds__((BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>::NT)
             // one right after the barrier: measured, each way is a few per cent better in its case.
             auto issue_copies = [&]() {
                 const unsigned saved_m0 = lds_copy_begin();
-                if constexpr (Q_BY_S) issue_q(nb + C::LA);
-                if constexpr (BV) issue_bias(nb + C::LA);
-                if constexpr (DO_BY_S) issue_do(t + C::LA);
+                if constexpr (IN) {
+                    settle_ptrs(run_rows, run_stat, run_bias);
+                    if constexpr (Q_BY_S) issue_next_q(nb + C::LA);
+                    if constexpr (BV) issue_next_bias(nb + C::LA);
+                    if constexpr (DO_BY_S) issue_next_do(t + C::LA);
+                } else {
+                    if constexpr (Q_BY_S) issue_q(nb + C::LA);
+                    if constexpr (BV) issue_bias(nb + C::LA);
+                    if constexpr (DO_BY_S) issue_do(t + C::LA);
+                }
                 lds_copy_end(saved_m0);
             };
             const unsigned char* bt_lds = ring_lds + ((nb - mb_first) % C::RING) * C::BT_BYTES;
-            const float* lse_lds = reinterpret_cast<const float*>(smem + C::OFF_LSE) + (nb % C::NQB) * BMI;
+            const float* lse_lds = reinterpret_cast<const float*>(smem + C::OFF_LSE) + (IN ? (unsigned)nb % C::NQB : nb % C::NQB) * (C::STAT_BYTES / 4);
             // inputs of P: LSE of 4 consecutive rows and the bias of those rows at this lane's key
             f32x4 lse_in[NSUB][4];
             BiasQuad<BIAS> bias_in[NSUB][4];
@@ -804,7 +872,7 @@ __global__ __launch_bounds__((BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>::NT)
             // by term; interior blocks fold everything into one exponent. ----
             auto make_p = [&]() {
                 const int m0 = nb * BMI;
-                const bool need_mask = (m0 + BMI > M) || (n0 + BN > N) || (CAUSAL && m0 < n0 + BN - 1);
+                const bool need_mask = !IN && ((m0 + BMI > M) || (n0 + BN > N) || (CAUSAL && m0 < n0 + BN - 1));
                 const float mf0 = (float)(m0 + 4 * g);  // ALiBi: first row of this lane's registers, as a float
                 float* p_out = p_lds + (nb & 1) * (C::P_BYTES / 4);
                 auto p_step = [&](auto masked_tag) {
@@ -846,8 +914,12 @@ __global__ __launch_bounds__((BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>::NT)
                         }
                     }
                 };
-                if (need_mask) p_step(std::true_type{});
-                else p_step(std::false_type{});
+                if constexpr (IN) {
+                    p_step(std::false_type{});
+                } else {
+                    if (need_mask) p_step(std::true_type{});
+                    else p_step(std::false_type{});
+                }
             };
             if constexpr (TB != 0 && !BV) {
                 if (nb < n_mblocks) load_bias_scalar(nb, ring_lds + ((nb - mb_first) % C::RING) * C::BT_BYTES);
@@ -861,27 +933,27 @@ __global__ __launch_bounds__((BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>::NT)
                 }
                 issue_copies();  // behind the reads, whose round trip they cover
                 if constexpr (!PRELOAD) load_p_inputs();
-                if (nb < n_mblocks) make_p();
+                if (IN || nb < n_mblocks) make_p();
                 if constexpr (PRELOAD) __builtin_amdgcn_sched_barrier(0);
-                load_cols(do_tile(t), a_cols);
-                load_rows(q_tile(nb + 1), a_rows);  // lands while the first product runs
+                load_cols((IN ? do_tile_in(t) : do_tile(t)), a_cols);
+                load_rows((IN ? q_tile_in(nb + 1) : q_tile(nb + 1)), a_rows);  // lands while the first product runs
                 if constexpr (PRELOAD) __builtin_amdgcn_sched_barrier(0);
                 // dV^T += dO(t)^T P(t), then the scores of block nb + 1 for the next step
-                if (t >= mb_first && t < n_mblocks) mma_cols(a_cols, op_cur);
-                if (nb + 1 < n_mblocks) mma_rows(a_rows, sacc);
+                if (IN || (t >= mb_first && t < n_mblocks)) mma_cols(a_cols, op_cur);
+                if (IN || nb + 1 < n_mblocks) mma_rows(a_rows, sacc);
             } else {
                 T8 a_cols[NA], a_rows[NR];
                 if constexpr (TB == 0) issue_copies();
-                load_cols(do_tile(t), a_cols);
-                load_rows(q_tile(nb), a_rows);
+                load_cols((IN ? do_tile_in(t) : do_tile(t)), a_cols);
+                load_rows((IN ? q_tile_in(nb) : q_tile(nb)), a_rows);
                 if constexpr (PRELOAD) {
                     load_p_inputs();
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 if constexpr (TB != 0) issue_copies();
                 // dV^T += dO(t)^T P(t) first: its operands do not depend on this step
-                if (t >= mb_first && t < n_mblocks) mma_cols(a_cols, op_cur);
-                if (nb < n_mblocks) {
+                if (IN || (t >= mb_first && t < n_mblocks)) mma_cols(a_cols, op_cur);
+                if (IN || nb < n_mblocks) {
                     mma_rows(a_rows, sacc);
                     if constexpr (!PRELOAD) load_p_inputs();
                     make_p();
@@ -899,8 +971,30 @@ __global__ __launch_bounds__((BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>::NT)
             else wait_vmcnt<OPS*(C::LA - 1)>();
             lds_barrier();
         };
+        // interior steps: t >= mb_first (block t is accumulated), the copied blocks up to t + 1 + LA are
+        // whole, and block t + 1 lies below the causal diagonal of every key of the tile
+        // Both roles run steps mb_first - 1 .. n_mblocks, whatever part of them is interior.
+        const int t_end = n_mblocks + 1;
+        int t_in = mb_first, t_out = n_full - C::LA - 1;
+        if (CAUSAL) t_in = (n0 + BN - 1 + BMI - 1) / BMI - 1 > t_in ? (n0 + BN - 1 + BMI - 1) / BMI - 1 : t_in;
+        if (n0 + BN > N || (TB != 0 && !BV)) t_out = t_in;  // a ragged key tile, bias element by element: no interior
+        t_in = t_in < t_end ? t_in : t_end;
+        t_out = t_out < t_in ? t_in : (t_out < t_end ? t_out : t_end);
+        if (!IN_LOOPS) t_in = t_out = t_end;  // one general loop
+        int t = mb_first - 1;
 #pragma unroll 1
-        for (int t = mb_first - 1; t <= n_mblocks; t++) s_step(t);
+        for (; t < t_in; t++) s_step(t, std::false_type{});
+        if constexpr (IN_LOOPS) {
+            if (t_in < t_out) {
+                run_start(qp, p.sq.s, lsep, t_in + 1 + C::LA, t_in + 1 + C::LA);
+#pragma unroll 1
+                for (; t < t_out; t++) s_step(t, std::true_type{});
+            }
+        }
+        if constexpr (IN_LOOPS) {
+#pragma unroll 1
+            for (; t < t_end; t++) s_step(t, std::false_type{});
+        }
         };
         if (TB != 0 && bias_vec) s_loop(std::true_type{});
         else s_loop(std::false_type{});
@@ -934,19 +1028,25 @@ __global__ __launch_bounds__((BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>::NT)
         // copies per step; the dBias stores that may sit between them in the queue are not
         // counted, which only makes the wait at the end of a step stricter
         constexpr int COPIES = ((Q_BY_S ? 0 : 1) + (DO_BY_S ? 0 : 1)) * (C::QD + 1);
-#pragma unroll 1
-        for (int t = mb_first - 1; t <= n_mblocks; t++) {
+        auto dp_step = [&](int t, auto in_tag) {
+            // IN: an interior step: blocks t - 1 .. t + LA are whole and in range
+            constexpr bool IN = decltype(in_tag)::value;
             auto issue_copies = [&]() {
                 if constexpr (COPIES > 0) {
                     const unsigned saved_m0 = lds_copy_begin();
-                    if constexpr (!Q_BY_S) issue_q(t + 1 + C::LA);
-                    if constexpr (!DO_BY_S) issue_do(t + C::LA);
+                    if constexpr (IN) {
+                        settle_ptrs(run_rows, run_stat, run_bias);
+                        issue_next_do(t + C::LA);
+                    } else {
+                        if constexpr (!Q_BY_S) issue_q(t + 1 + C::LA);
+                        if constexpr (!DO_BY_S) issue_do(t + C::LA);
+                    }
                     lds_copy_end(saved_m0);
                 }
             };
-            const bool live = t >= mb_first && t < n_mblocks;
+            const bool live = IN || (t >= mb_first && t < n_mblocks);
             const int m0 = t * BMI;
-            const float* delta_lds = reinterpret_cast<const float*>(smem + C::OFF_DELTA) + ((t < 0 ? 0 : t) % C::NDOB) * BMI;
+            const float* delta_lds = reinterpret_cast<const float*>(smem + C::OFF_DELTA) + (IN ? (unsigned)t % C::NDOB : (t < 0 ? 0 : t) % C::NDOB) * (C::STAT_BYTES / 4);
             const float* p_in = p_lds + (t & 1) * (C::P_BYTES / 4);
             T8 a_cols[NA], a_rows[NR];
             f32x4 del_in[NSUB][4], p_vals[NSUB][4];
@@ -961,11 +1061,11 @@ __global__ __launch_bounds__((BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>::NT)
             };
             if constexpr (TB == 0) issue_copies();
             // operands of both products up front: Q(t-1)^T for dK, the rows of dO(t) for dP
-            if constexpr (C::DEFER_DK) load_cols(q_tile(t - 1), a_cols);
-            load_rows(do_tile(t), a_rows);
+            if constexpr (C::DEFER_DK) load_cols((IN ? q_tile_in(t - 1) : q_tile(t - 1)), a_cols);
+            load_rows((IN ? do_tile_in(t) : do_tile(t)), a_rows);
             if constexpr (PRELOAD && TB == 0) __builtin_amdgcn_sched_barrier(0);
             if constexpr (TB != 0) issue_copies();  // behind the reads, whose round trip they cover
-            if (C::DEFER_DK && t - 1 >= mb_first) mma_cols(a_cols, op_cur);  // dK^T += Q(t-1)^T dS(t-1)
+            if (C::DEFER_DK && (IN || t - 1 >= mb_first)) mma_cols(a_cols, op_cur);  // dK^T += Q(t-1)^T dS(t-1)
             if (live) {
                 f32x16 sacc[NSUB];
                 if constexpr (PRELOAD) {
@@ -1015,7 +1115,7 @@ __global__ __launch_bounds__((BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>::NT)
                         if constexpr (DB_FAST) {
                             // rows past M: m0 * row bytes alone is past the view only if the view is
                             // tight, so the row test is explicit
-                            const int off = m < M ? db_off[it] + m0 * db_row_bytes : (int)0x80000000;
+                            const int off = (IN || m < M) ? db_off[it] + m0 * db_row_bytes : (int)0x80000000;
                             buf_store16(db_rsrc, v, off);
                         } else if (m < M && nn < N) {
                             E* dst = dbp + (int64_t)m * p.sdbias.m + (int64_t)nn * p.sdbias.n;
@@ -1031,12 +1131,32 @@ __global__ __launch_bounds__((BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>::NT)
                     }
                 }
                 if constexpr (!C::DEFER_DK) {  // dK^T += Q(t)^T dS(t)
-                    load_cols(q_tile(t), a_cols);
+                    load_cols((IN ? q_tile_in(t) : q_tile(t)), a_cols);
                     mma_cols(a_cols, op_cur);
                 }
             }
             if constexpr (COPIES > 0) wait_vmcnt<COPIES*(C::LA - 1)>();
             lds_barrier();
+        };
+        // interior steps: block t - 1 was accumulated into dS (t - 1 >= mb_first) and the copied block t + LA is whole
+        const int t_end = n_mblocks + 1;
+        int t_in = mb_first + 1, t_out = n_full - C::LA;
+        t_in = t_in < t_end ? t_in : t_end;
+        t_out = t_out < t_in ? t_in : (t_out < t_end ? t_out : t_end);
+        if (!IN_LOOPS) t_in = t_out = t_end;  // one general loop
+        int t = mb_first - 1;
+#pragma unroll 1
+        for (; t < t_in; t++) dp_step(t, std::false_type{});
+        if constexpr (IN_LOOPS) {
+            if (t_in < t_out) {
+                run_start(dop, p.sdo.s, deltap, t_in + C::LA, 0);
+#pragma unroll 1
+                for (; t < t_out; t++) dp_step(t, std::true_type{});
+            }
+        }
+        if constexpr (IN_LOOPS) {
+#pragma unroll 1
+            for (; t < t_end; t++) dp_step(t, std::false_type{});
         }
         };
         if constexpr (DB_VIA_LDS) {

@@ -200,6 +200,17 @@ __device__ __forceinline__ uint64_t uniform_ptr(const void* p) {
     asm volatile("s_nop 4" : "+s"(lo), "+s"(hi));
     return ((uint64_t)hi << 32) | lo;
 }
+// The same for up to three addresses that a loop keeps and advances in scalar registers: one wait
+// for all of them, in place, so that no copy of an address is made per use.
+__device__ __forceinline__ void settle_ptrs(uint64_t& a, uint64_t& b, uint64_t& c) {
+    unsigned r[6] = {(unsigned)a, (unsigned)(a >> 32), (unsigned)b, (unsigned)(b >> 32), (unsigned)c, (unsigned)(c >> 32)};
+#pragma unroll
+    for (int i = 0; i < 6; i++) r[i] = __builtin_amdgcn_readfirstlane(r[i]);
+    asm volatile("s_nop 4" : "+s"(r[0]), "+s"(r[1]), "+s"(r[2]), "+s"(r[3]), "+s"(r[4]), "+s"(r[5]));
+    a = ((uint64_t)r[1] << 32) | r[0];
+    b = ((uint64_t)r[3] << 32) | r[2];
+    c = ((uint64_t)r[5] << 32) | r[4];
+}
 // between lds_copy_begin() and lds_copy_end(): 16 bytes per lane from base + voff to lds_addr + 16 l
 __device__ __forceinline__ void lds_copy16(uint64_t base, unsigned voff, unsigned lds_addr) {
     asm volatile(

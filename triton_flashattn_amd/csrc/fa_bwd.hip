@@ -149,9 +149,15 @@ __global__ __launch_bounds__(256, (StreamCfg<D, stream_kind(BIAS)>::MIN_BLOCKS))
     // One step of the K/V stream.  Interior steps (every key in range and visible to every row of
     // the work-group) run with STEP_MASKED = false: no range checks, no mask arithmetic.  BV: the
     // bias slices come by copy (rows that allow aligned 16-byte chunks), else element by element.
-    auto kv_step = [&](int k, auto step_tag, auto bv_tag) {
+    // LEAN: the copies of the step need no clamps (KeyStream::issue_ahead_lean).
+    auto kv_step = [&](int k, auto step_tag, auto bv_tag, auto lean_tag) {
         constexpr bool STEP_MASKED = decltype(step_tag)::value;
         constexpr bool BV = decltype(bv_tag)::value;
+        constexpr bool LEAN = decltype(lean_tag)::value;
+        auto issue_ahead = [&]() {
+            if constexpr (LEAN) ks_.template issue_ahead_lean<BV>(k);
+            else ks_.template issue_ahead<BV>(k);
+        };
         const int n0 = k * BK;
         ks_.template begin_step<BV>(k);
         const unsigned k_tile = ks_.k_addr(k), v_tile = ks_.v_addr(k);  // operand reads by address
@@ -164,7 +170,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, stream_kind(BIAS)>::MIN_BLOCKS))
             __builtin_amdgcn_sched_barrier(0);  // keep the blocks apart
             // blocks entirely above this wave's diagonal or past the last key contribute nothing
             if (STEP_MASKED && ((CAUSAL && n0 + nh > mw + 31) || n0 + nh >= N)) {
-                if (nb == 0) ks_.template issue_ahead<BV>(k);  // every wave issues its copies in every step
+                if (nb == 0) issue_ahead();  // every wave issues its copies in every step
                 continue;
             }
             const bool need_mask = STEP_MASKED && ((n0 + nh + 32 > N) || (CAUSAL && n0 + nh + 31 > mw));
@@ -212,7 +218,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, stream_kind(BIAS)>::MIN_BLOCKS))
                 T8 a = SW::template row8_at<T8>(v_tile + rows_l, nh, ks);
                 dp = mfma32(a, doreg[ks], dp);
             }
-            if (nb == 0) ks_.template issue_ahead<BV>(k);  // in the shadow of the MFMAs just issued
+            if (nb == 0) issue_ahead();  // in the shadow of the MFMAs just issued
 
             // ---- P = 2^(S*scale + bias - LSE), dS = P (dP - delta) (flash_attention.py:497-517).
             // Masked tiles follow the reference's additive -1e6 arithmetic term by term.
@@ -292,7 +298,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, stream_kind(BIAS)>::MIN_BLOCKS))
                     dq_acc[db] = mfma32(a, dsb[kk], dq_acc[db]);
                 }
             }
-            if (FROM_DS && nb == 0) ks_.template issue_ahead<BV>(k);  // in the shadow of the MFMAs just issued
+            if (FROM_DS && nb == 0) issue_ahead();  // in the shadow of the MFMAs just issued
         }
     };
 
@@ -303,10 +309,18 @@ __global__ __launch_bounds__(256, (StreamCfg<D, stream_kind(BIAS)>::MIN_BLOCKS))
     auto run = [&](auto bv_tag) {
         constexpr bool BV = decltype(bv_tag)::value;
         ks_.template prologue<BV>();
+        // the leading fast steps whose copies stay inside the tensors issue them without clamps
+        const int n_lean = (BV || TB == 0) ? ks_.lean_steps(n_fast, m0 + BM) : 0;
+        int k = 0;
+        if (n_lean > 0) {
+            ks_.run_start(C::LA, C::NBS - 1);
 #pragma unroll 1
-        for (int k = 0; k < n_fast; k++) kv_step(k, std::false_type{}, bv_tag);
+            for (; k < n_lean; k++) kv_step(k, std::false_type{}, bv_tag, std::true_type{});
+        }
 #pragma unroll 1
-        for (int k = n_fast; k < n_steps; k++) kv_step(k, std::true_type{}, bv_tag);
+        for (; k < n_fast; k++) kv_step(k, std::false_type{}, bv_tag, std::false_type{});
+#pragma unroll 1
+        for (; k < n_steps; k++) kv_step(k, std::true_type{}, bv_tag, std::false_type{});
     };
     if (FROM_DS || (TB != 0 && p.bias_vec)) run(std::true_type{});
     else run(std::false_type{});

@@ -377,6 +377,14 @@ template <typename T, int D, int BIAS, bool WITH_V = true> struct KeyStream {
     unsigned lean_x16, lean_rk, lean_rv;  // ((l % 32) ^ (g << 2)) * 16, byte offsets of row g of K and of V
     int wave_s;                           // wave index (scalar)
     unsigned lds_kv, lds_bias;  // LDS addresses (scalar) of the K slots and of this wave's bias ring
+    // Lean steps (issue_ahead_lean): every row they copy exists, so the copies need no clamps and walk
+    // the keys with running 64-bit addresses in scalar registers, one add per step: the K and V rows
+    // of the next step to copy, and this wave's bias rows at the first key of the next slice to copy.
+    uint64_t run_k, run_v, run_b;
+    // byte offset of this lane's chunk in bias copy `it`: with 1- and 2-byte elements the copies of a
+    // slice are whole groups of rows apart with the same chunk order, so one offset and a stride do
+    static constexpr int NBOFF = C::ES == 4 ? C::BCH : 1;
+    unsigned lean_boff[NBOFF];
     // chunk index of copy i of this wave (scalar)
     __device__ __forceinline__ int copy_idx(int i) const { return LEAN ? (wave_s * C::KD + i) % C::NKD : c_idx[i]; }
 
@@ -445,7 +453,11 @@ template <typename T, int D, int BIAS, bool WITH_V = true> struct KeyStream {
                 vo = v_off[i];
             }
             if (!full) {
-                const int c = ci * 64 + lane;
+                // (rare: the lane index passes through an empty asm so that these per-lane values are
+                // formed here and not kept in registers across the loops)
+                int lane_here = lane;
+                asm volatile("" : "+v"(lane_here));
+                const int c = ci * 64 + lane_here;
                 int row = c / C::CPR;
                 const int src = (c % C::CPR) ^ SW::f(row);
                 row = row < N - n0 ? row : N - 1 - n0;
@@ -476,6 +488,70 @@ template <typename T, int D, int BIAS, bool WITH_V = true> struct KeyStream {
                 lds_copy16(base, (unsigned)(((int64_t)m * sbm + n) * C::ES), dst + it * 1024);
             }
         }
+    }
+    // Points the running addresses at K/V step `k_kv` and bias slice `k_b` (the next ones a lean step issues).
+    __device__ __forceinline__ void run_start(int k_kv, int k_b) {
+        run_k = uniform_ptr(kp + (int64_t)k_kv * C::BK * sk);
+        run_v = uniform_ptr(vp + (int64_t)k_kv * C::BK * sv);
+        run_b = 0;
+        if constexpr (C::ES != 0) {
+            run_b = uniform_ptr(reinterpret_cast<const unsigned char*>(bp) + ((int64_t)mw * sbm + (int64_t)k_b * C::BK) * C::ES);
+            // (2-byte elements: a copy covers 16 rows and the chunk order depends on (row / 4) % 4;
+            // 1-byte elements: one copy per slice)
+            static_assert(C::ES == 4 || C::ES == 2 || C::BCH == 1, "chunk order repeats from copy to copy");
+#pragma unroll
+            for (int it = 0; it < NBOFF; it++) {
+                const int c = it * 64 + lane;
+                const int row = c / C::BCPR;
+                lean_boff[it] = (unsigned)(((int64_t)row * sbm + ((c % C::BCPR) ^ C::bswz(row)) * C::EPC) * C::ES);
+            }
+        }
+    }
+    // issue_ahead for a step whose copies (K/V rows of step k + LA, bias slice of step k + NBS - 1, all
+    // 32 rows of this wave) lie wholly inside the tensors; run_start() was called for the first such step
+    template <bool BV> __device__ __forceinline__ void issue_ahead_lean(int k) {
+        const unsigned saved_m0 = lds_copy_begin();
+        settle_ptrs(run_k, run_v, run_b);
+        const unsigned k_dst = lds_kv + (unsigned)((k + C::LA) % C::NKV) * C::STEP_BYTES;
+        const unsigned v_dst = k_dst + C::NKV * C::STEP_BYTES;
+#pragma unroll
+        for (int i = 0; i < C::KD; i++) {
+            const int ci = copy_idx(i);
+            unsigned ko, vo;
+            if constexpr (LEAN) {
+                const int r0 = (64 / C::CPR) * ci;
+                const unsigned x = lean_x16 ^ (unsigned)((((r0 & 3) << 2) | ((r0 >> 2) & 3)) << 4);
+                ko = x + lean_rk + (unsigned)(r0 * (int)sk * 2);
+                vo = x + lean_rv + (unsigned)(r0 * (int)sv * 2);
+            } else {
+                ko = k_off[i];
+                vo = v_off[i];
+            }
+            lds_copy16(run_k, ko, k_dst + ci * 1024);
+            if constexpr (WITH_V) lds_copy16(run_v, vo, v_dst + ci * 1024);
+        }
+        run_k += (uint64_t)(C::BK * 2) * (uint64_t)sk;
+        run_v += (uint64_t)(C::BK * 2) * (uint64_t)sv;
+        if constexpr (BV && C::ES != 0) {
+            const unsigned dst = lds_bias + (unsigned)((k + C::NBS - 1) % C::NBS) * C::BSLOT;
+#pragma unroll
+            for (int it = 0; it < C::BCH; it++) {
+                const unsigned off = C::ES == 4 ? lean_boff[it < NBOFF ? it : 0]
+                                                : lean_boff[0] + (unsigned)(it * (64 / C::BCPR) * (int)sbm * C::ES);
+                lds_copy16(run_b, off, dst + it * 1024);
+            }
+            run_b += C::BK * C::ES;
+        }
+        lds_copy_end(saved_m0);
+    }
+    // lean steps a kernel may run from step 0: those whose copies stay inside N keys (and, with a bias, whose
+    // work-group has all of its rows), at most `limit`
+    __device__ __forceinline__ int lean_steps(int limit, int wg_rows_end) const {
+        constexpr int AHEAD = (C::ES != 0 && C::NBS - 1 > C::LA) ? C::NBS - 1 : C::LA;
+        int n = N / C::BK - AHEAD;
+        if (C::ES != 0 && wg_rows_end > M) n = 0;
+        n = n < limit ? n : limit;
+        return n < 0 ? 0 : n;
     }
     // Before the first step, in the order the steps assume: the first bias slices, then K/V of a
     // step followed by the bias slice issued in the same step.  BV: the bias slices come by copy.

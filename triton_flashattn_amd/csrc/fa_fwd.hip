@@ -112,9 +112,15 @@ __global__ __launch_bounds__(256, (StreamCfg<D, fwd_stream_kind(BIAS)>::MIN_BLOC
     // One step of the K/V stream.  Interior steps (every key in range and visible to every row of
     // the work-group) run with STEP_MASKED = false: no range checks, no mask arithmetic.  BV: the
     // bias slices come by copy (rows that allow aligned 16-byte chunks), else element by element.
-    auto kv_step = [&](int k, auto step_tag, auto bv_tag) {
+    // LEAN: the copies of the step need no clamps (KeyStream::issue_ahead_lean).
+    auto kv_step = [&](int k, auto step_tag, auto bv_tag, auto lean_tag) {
         constexpr bool STEP_MASKED = decltype(step_tag)::value;
         constexpr bool BV = decltype(bv_tag)::value;
+        constexpr bool LEAN = decltype(lean_tag)::value;
+        auto issue_ahead = [&]() {
+            if constexpr (LEAN) ks_.template issue_ahead_lean<BV>(k);
+            else ks_.template issue_ahead<BV>(k);
+        };
         const int n0 = k * BK;
         ks_.template begin_step<BV>(k);
         const unsigned k_rows = ks_.k_addr(k) + rows_l, v_cols = ks_.v_addr(k) + cols_l;  // operand reads by address
@@ -136,7 +142,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, fwd_stream_kind(BIAS)>::MIN_BLOC
                     s_pre[nb] = mfma32(a, qreg[ks], s_pre[nb]);
                 }
             }
-            ks_.template issue_ahead<BV>(k);  // in the shadow of the MFMAs just issued
+            issue_ahead();  // in the shadow of the MFMAs just issued
         }
 #pragma unroll
         for (int nb = 0; nb < C::NH; nb++) {
@@ -144,7 +150,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, fwd_stream_kind(BIAS)>::MIN_BLOC
         __builtin_amdgcn_sched_barrier(0);  // keep the blocks apart
         // blocks entirely above this wave's diagonal or past the last key contribute nothing
         if (STEP_MASKED && ((CAUSAL && n0 + nh > mw + 31) || n0 + nh >= N)) {
-            if (nb == 0) ks_.template issue_ahead<BV>(k);  // every wave issues its copies in every step
+            if (nb == 0) issue_ahead();  // every wave issues its copies in every step
             continue;
         }
         const bool need_mask = STEP_MASKED && ((n0 + nh + 32 > N) || (CAUSAL && n0 + nh + 31 > mw));
@@ -161,7 +167,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, fwd_stream_kind(BIAS)>::MIN_BLOC
                 T8 a = SW::template row8_at<T8>(k_rows, nh, ks);
                 s = mfma32(a, qreg[ks], s);
             }
-            if (nb == 0) ks_.template issue_ahead<BV>(k);  // in the shadow of the MFMAs just issued
+            if (nb == 0) issue_ahead();  // in the shadow of the MFMAs just issued
         }
 
         // ---- online softmax step.  `masked` steps (ragged edge, causal diagonal) and a
@@ -285,10 +291,18 @@ __global__ __launch_bounds__(256, (StreamCfg<D, fwd_stream_kind(BIAS)>::MIN_BLOC
     auto run = [&](auto bv_tag) {
         constexpr bool BV = decltype(bv_tag)::value;
         ks_.template prologue<BV>();
+        // the leading fast steps whose copies stay inside the tensors issue them without clamps
+        const int n_lean = (BV || TB == 0) ? ks_.lean_steps(n_fast, m0 + BM) : 0;
+        int k = 0;
+        if (n_lean > 0) {
+            ks_.run_start(C::LA, C::NBS - 1);
 #pragma unroll 1
-        for (int k = 0; k < n_fast; k++) kv_step(k, std::false_type{}, bv_tag);
+            for (; k < n_lean; k++) kv_step(k, std::false_type{}, bv_tag, std::true_type{});
+        }
 #pragma unroll 1
-        for (int k = n_fast; k < n_steps; k++) kv_step(k, std::true_type{}, bv_tag);
+        for (; k < n_fast; k++) kv_step(k, std::false_type{}, bv_tag, std::false_type{});
+#pragma unroll 1
+        for (; k < n_steps; k++) kv_step(k, std::true_type{}, bv_tag, std::false_type{});
     };
     if (TB != 0 && p.bias_vec) run(std::true_type{});
     else run(std::false_type{});

@@ -9,7 +9,10 @@
  *                /root/reference/flash_attention.py:688-763
  * Like them, the library owns no memory: every buffer (including the backward workspace) is
  * allocated by the caller, every call only enqueues work on the stream it is given and returns
- * without synchronizing.  All entry points are re-entrant and keep no mutable global state.
+ * without synchronizing.  All entry points are re-entrant and keep no mutable global state, with
+ * one exception: fa_bwd_noalloc (at the end of this header) keeps its scratch in a static device
+ * array of the library, 8 MiB on every GPU it runs on, and a per-device cache of that array's
+ * address; calls of it that overlap on one GPU race on the array.
  *
  * Layouts (element strides, as the reference passes them, flash_attention.py:670-675):
  *   q, o, do, dq : (B, M, H, D)     k, v, dk, dv : (B, N, H, D)     the D stride must be 1
@@ -19,8 +22,11 @@
  * (FA_ERR_LAYOUT otherwise; FA_ERR_HEAD_STRIDE for a D stride other than 1); bias/dbias have no
  * alignment requirement, but only rows with unit N stride and 16-byte aligned row starts that are
  * whole 16-byte chunks, or whose row stride covers the last chunk (N * element size rounded up to 16
- * bytes: a padded row pitch or a column slice of a wider tensor; the bytes behind the last key of
- * every row are then read, never written), take the fast path.  With FA_MI355_VERBOSE set in the
+ * bytes: a padded row pitch or a column slice of a wider tensor), take the fast path.  On that path
+ * the bytes behind the last key of EVERY row, up to the end of its 16-byte chunk, are read (never
+ * written), the last row of the last (batch, head) slice included: the caller guarantees that the
+ * chunk holding the last element of the tensor lies inside the allocation (a row-strided view whose
+ * last row ends the allocation does not qualify and must be copied to a padded pitch first).  With FA_MI355_VERBOSE set in the
  * environment the library says on stderr, once per process, when a bias or dbias misses that path
  * and is read or written element by element (several times slower).
  */
@@ -127,7 +133,7 @@ int fa_fwd(const fa_fwd_args *args, void *stream);
 size_t fa_bwd_workspace_bytes(const fa_problem *p);
 
 /* Scratch with which fa_fwd splits the keys of a query tile between several work-groups and merges
- * their softmaxes (the outputs of the shares in the element type of q, and their LSEs); 0 when the
+ * their softmaxes (the outputs of the shares in fp32, and their LSEs); 0 when the
  * problem has enough query tiles to fill the GPU, or is causal.  No counterpart in the reference (its grid is one program
  * per query tile, flash_attention.py:666).  The workspace is optional: without it fa_fwd runs one
  * work-group per query tile, with the same results up to fp32 rounding of the merge. */
@@ -167,7 +173,10 @@ int fa_bwd_stages(const fa_bwd_args *args, void *stream, int stages);
  * B * H * M nor B * H * max(N, 4) may exceed FA_NOALLOC_MAX_ROWS (FA_ERR_TOO_LARGE
  * otherwise).  The call allocates and frees nothing.  All calls on one GPU share the array:
  * calls that may overlap on one GPU (different streams, different threads) race on it; on one
- * stream they are ordered and safe.  Results are bit-identical to fa_bwd. */
+ * stream they are ordered and safe.  Results are bit-identical to fa_bwd.
+ * The first call on a device asks the runtime for the array's address on that device
+ * (hipGetSymbolAddress, which may load the library's code object): make one call on every device
+ * before any stream capture; later calls only read the cached address. */
 #define FA_NOALLOC_MAX_ROWS (1 << 20)
 int fa_bwd_noalloc(const fa_bwd_args *args, void *stream);
 

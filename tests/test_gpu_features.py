@@ -311,8 +311,9 @@ def test_split_forward_equals_unsplit_forward(gpu_device):
         torch.cuda.synchronize()
         outs.append((o, lse))
     (o1, l1), (o2, l2) = outs
-    assert not torch.equal(o1, o2) or True        # they may differ in the last bit
-    assert (o1.float() - o2.float()).abs().max().item() <= 2 ** -6 * o2.float().abs().max().item()
+    # the shares stay in fp32 and the merge rounds once: fp32 reassociation can move a result across a
+    # rounding boundary, so the two runs differ by one bf16 step (at most 2^-7 of the value) and no more
+    assert (o1.float() - o2.float()).abs().max().item() <= 2 ** -7 * o2.float().abs().max().item()
     assert torch.allclose(l1, l2, atol=1e-4, rtol=1e-6)
 
 
@@ -330,3 +331,48 @@ def test_library_operator_matches_the_function(gpu_device):
         assert torch.equal(got, want[n]), n
     torch.library.opcheck(torch.ops.fa_mi355.attention_fwd.default, (q, k, v, bias.detach(), True, 0.125),
                           test_utils=("test_schema", "test_faketensor"))
+
+
+# ---------------------------------------------------------------- autocast and torch.compile on the GPU
+def test_autocast_region_runs_the_kernels_on_float32_inputs(gpu_device):
+    """fp32 q, k, v inside torch.autocast('cuda', bfloat16): the kernels run in bf16 (as the matrix
+    products of an eager attention would), the output is bf16, the gradients come back in fp32, and
+    everything agrees with the oracle on the bf16-rounded inputs."""
+    B, M, N, H, D = 2, 150, 210, 2, 64
+    q, k, v, do, bias = make_inputs(gpu_device, B, M, N, H, D, torch.float32, "f32", seed=71)
+    ql, kl, vl = (t.detach().clone().requires_grad_(True) for t in (q, k, v))
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        out = flash_attention_fn(ql, kl, vl, bias, False)
+    assert out.dtype == torch.bfloat16
+    out.backward(do.bfloat16())
+    assert ql.grad.dtype == torch.float32 and kl.grad.dtype == torch.float32 and bias.grad.dtype == torch.float32
+    ref = run_oracle(q.bfloat16(), k.bfloat16(), v.bfloat16(), do.bfloat16(), bias, False)
+    check({"out": out.detach(), "dq": ql.grad, "dk": kl.grad, "dv": vl.grad, "dbias": bias.grad}, ref, "autocast")
+    # outside a region fp32 inputs are refused as before
+    with pytest.raises(TypeError):
+        flash_attention_fn(q, k, v, None, False)
+
+
+def test_compiled_call_of_the_library_operator_runs_the_kernels(gpu_device):
+    """torch.compile (backend aot_eager: traced with fake tensors, functionalised, differentiated ahead of
+    time, no code generation) around flash_attention_op: the compiled forward and backward call the HIP
+    kernels and return what the eager function returns, bit for bit, and what the oracle returns
+    within the tolerances."""
+    B, M, N, H, D = 1, 257, 257, 2, 64
+    q, k, v, do, bias = make_inputs(gpu_device, B, M, N, H, D, torch.bfloat16, "bf16", seed=72)
+    want = run_ours(q, k, v, do, bias, True)
+
+    def block(q, k, v, b):
+        return flash_attention_op(q * 1.0, k, v, b, True) * 1.0   # something around the operator to trace
+
+    compiled = torch.compile(block, backend="aot_eager", fullgraph=True)
+    q2, k2, v2 = (t.detach().clone().requires_grad_(True) for t in (q, k, v))
+    b2 = bias.detach().clone().requires_grad_(True)
+    out = compiled(q2, k2, v2, b2)
+    out.backward(do)
+    torch.cuda.synchronize()
+    assert torch.equal(out, want["out"])
+    got = {"out": out.detach(), "dq": q2.grad, "dk": k2.grad, "dv": v2.grad, "dbias": b2.grad}
+    for n in ("dq", "dk", "dv", "dbias"):
+        assert torch.equal(got[n], want[n]), n
+    check(got, run_oracle(q, k, v, do, bias, True), "compiled")

@@ -303,6 +303,43 @@ def test_layout_rule_matches_the_c_side():
     assert fa_mod._kernel_layout_ok(torch.zeros(1, 4, 1, 16, dtype=torch.bfloat16))
 
 
+def test_padded_bias_rows_must_end_inside_the_storage():
+    """Rows that end inside a 16-byte chunk are fetched to the end of that chunk, so the chunk of the last
+    row has to exist: a column slice of a wider tensor qualifies, a row-strided view whose last row ends
+    the allocation does not (it is copied to a padded pitch instead)."""
+    N = 100   # 200 bytes per bf16 row: the last chunk is half used
+    wide = torch.zeros(1, 2, 7, 128, dtype=torch.bfloat16)
+    assert fa_mod._bias_rows_ok(wide[..., :N])                      # the other columns follow every row
+    big = torch.zeros(1, 1, 7, N, dtype=torch.bfloat16)
+    strided = big[:, :, ::2, :]                                      # 4 rows, 400 bytes apart; row 6 ends the storage
+    assert strided.stride(2) * 2 >= 208 and not fa_mod._bias_rows_ok(strided)
+    assert fa_mod._bias_rows_ok(big[:, :, :6:2, :])                  # its last row is followed by row 5
+    out = fa_mod._bias_kernel_layout(strided)
+    assert out is not strided and fa_mod._bias_rows_ok(out) and torch.equal(out, strided)
+    exact = torch.zeros(1, 1, 7, 96, dtype=torch.bfloat16)           # whole chunks: nothing is read past a row
+    assert fa_mod._bias_rows_ok(exact[:, :, ::2, :])
+
+
+def test_hip_backend_checks_shapes_before_launching():
+    """The launchers may be called directly (as in the reference): tensors that disagree with the extents
+    taken from q and k are refused, not read out of bounds."""
+    q, k, v = _qkv(D=16)
+    lse = torch.zeros(2, 2, 6)
+    chk = fa_mod._HipBackend._check_shapes
+    chk(q, k, v, lse, None, False, like_q=[("o", torch.zeros_like(q))])
+    with pytest.raises(ValueError, match="v has shape"):
+        chk(q, k, v[..., :8], lse, None, False)
+    with pytest.raises(ValueError, match="v has shape"):
+        chk(q, k, v[:, :5], lse, None, False)
+    with pytest.raises(ValueError, match="o has shape"):
+        chk(q, k, v, lse, None, False, like_q=[("o", torch.zeros(2, 6, 2, 32))])
+    with pytest.raises(ValueError, match="lse"):
+        chk(q, k, v, torch.zeros(2, 6, 2), None, False)
+    with pytest.raises(ValueError, match="dbias has shape"):
+        chk(q, k, v, lse, torch.zeros(2, 2, 6, 9), False, dbias=torch.zeros(2, 2, 1, 9))
+    chk(q, k, v, lse, torch.zeros(2), True, dbias=torch.zeros(2))      # ALiBi: H slopes and their gradients
+
+
 # ---------------------------------------------------------------- C ABI surface (no launches)
 def _declared_functions():
     text = open(os.path.join(ROOT, "include", "fa_mi355.h")).read()
@@ -336,7 +373,7 @@ def test_abi_status_codes_and_workspace():
     assert lib.fa_bwd_workspace_bytes(ctypes.byref(p)) == pad(rows * 4) + pad(2 * 3 * 50 * 4)   # delta + partial sums
     assert lib.fa_fwd_workspace_bytes(ctypes.byref(p)) == 0            # too few keys to split
     few = _native.FaProblem(B=1, H=32, M=1024, N=8192, D=128, dtype=_native.FA_BF16, bias_dtype=3, causal=0, sm_scale=0.1)
-    assert lib.fa_fwd_workspace_bytes(ctypes.byref(few)) == pad(2 * 32 * 1024 * 128 * 2) + pad(2 * 32 * 1024 * 4)  # two shares
+    assert lib.fa_fwd_workspace_bytes(ctypes.byref(few)) == pad(2 * 32 * 1024 * 128 * 4) + pad(2 * 32 * 1024 * 4)  # two fp32 shares
     few.causal, few.N = 1, 1024
     assert lib.fa_fwd_workspace_bytes(ctypes.byref(few)) == 0            # never when causal
     many = _native.FaProblem(B=2, H=16, M=4096, N=4096, D=128, dtype=_native.FA_BF16, bias_dtype=3, causal=0, sm_scale=0.1)

@@ -1,6 +1,7 @@
 """fa_bwd_noalloc (delta in the library's static device array, nothing allocated) against fa_bwd
 on the same inputs, through the C ABI: bit-identical outputs, two calls in a row, the second on
-a smaller problem (the array keeps the first call's contents), and the size limit."""
+a smaller problem (the array keeps the first call's contents), the oracle on one of them, free
+device memory unchanged by a call, and the size limit."""
 import ctypes
 
 import pytest
@@ -9,6 +10,7 @@ import torch
 import triton_flashattn_amd.flash_attention as fa_mod
 from triton_flashattn_amd import _native
 from triton_flashattn_amd.flash_attention import _flash_attn_fwd
+from oracle.attention_oracle import reference_grads
 
 pytestmark = pytest.mark.gpu
 
@@ -24,10 +26,19 @@ def _backward_both_ways(dev, B, M, N, H, D, dtype, bias_dtype, causal, seed):
     for noalloc in (False, True):
         dq, dk, dv = torch.full_like(q, 7.0), torch.full_like(k, 7.0), torch.full_like(v, 7.0)
         dbias = None if bias is None else torch.full_like(bias, 7.0)
+        torch.cuda.synchronize()
+        free_before = torch.cuda.mem_get_info(dev)[0]
         fa_mod._backend.bwd(do, q, k, v, o, bias, causal, sm_scale, lse, dq, dk, dv, dbias, noalloc=noalloc)
         torch.cuda.synchronize()
+        if noalloc and not first_call_on_device[0]:
+            # (the first call on a device may load the library's code object; no later one takes memory)
+            assert torch.cuda.mem_get_info(dev)[0] == free_before
+        first_call_on_device[0] = first_call_on_device[0] and not noalloc
         outs.append((dq, dk, dv, dbias))
-    return outs
+    return outs + [reference_grads(q, k, v, bias, do, causal)]
+
+
+first_call_on_device = [True]
 
 
 def test_noalloc_backward_matches_fa_bwd_twice(gpu_device):
@@ -37,13 +48,16 @@ def test_noalloc_backward_matches_fa_bwd_twice(gpu_device):
         (1, 130, 77, 3, 64, torch.bfloat16, torch.float32, False, 3),
     ]
     for case in cases:
-        ref, got = _backward_both_ways(gpu_device, *case)
+        ref, got, oracle = _backward_both_ways(gpu_device, *case)
         for name, a, b in zip(("dq", "dk", "dv", "dbias"), ref, got):
             if a is None:
                 assert b is None
                 continue
             assert torch.isfinite(b.float()).all(), (case, name)
             assert torch.equal(a, b), (case, name)
+            # and against the oracle: relative L2 error within the tolerance of the parity tests
+            want = oracle[name].to(b.device)
+            assert ((b.float() - want).norm() / want.norm()).item() <= 5e-2, (case, name)
 
 
 def test_noalloc_rejects_problems_beyond_its_scratch(gpu_device):

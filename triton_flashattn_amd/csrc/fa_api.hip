@@ -171,19 +171,35 @@ size_t partial_floats(const fa_problem& p) {
     return (size_t)p.B * p.H * ((size_t)p.N > tiles4 ? (size_t)p.N : tiles4);
 }
 
+// Compute units of the current device (looked up once per device; 256, an MI355X, when no device
+// can be asked: the size queries must also work where no GPU is present).
+int compute_units() {
+    static std::atomic<int> cached[fa::kMaxDevices];
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= fa::kMaxDevices) return 256;
+    int n = cached[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cached[dev].store(n, std::memory_order_relaxed);
+    }
+    return n;
+}
+
 // Keys of a query tile split between work-groups when the query tiles alone leave the GPU half empty
 // (fewer than two work-groups per CU): as many splits as it takes to get there, at most four, each
-// with at least 16 steps of the K/V stream.
+// with at least 16 steps of the K/V stream.  The answer depends on the current device (its CU
+// count): a size query and the launch it sizes must run with the same device current.
 struct FwdSplit {
     int n_splits, keys_per_split;
 };
 FwdSplit fwd_split(const fa_problem& p) {
     if (p.causal) return {1, 0};
     const int64_t wgs = (int64_t)((p.M + fa::fwd_block_m() - 1) / fa::fwd_block_m()) * p.B * p.H;
-    if (wgs >= 512) return {1, 0};
+    const int64_t full = 2 * (int64_t)compute_units();
+    if (wgs >= full) return {1, 0};
     const int bk = p.bias_dtype == FA_BIAS_NONE ? 64 : 32;  // keys per step of the forward kernel
     const int n_steps = (p.N + bk - 1) / bk;
-    int s = (int)(512 / wgs);
+    int s = (int)(full / wgs);
     s = s > 4 ? 4 : s;
     while (s > 1 && n_steps / s < 16) s--;
     if (s <= 1) return {1, 0};
@@ -193,7 +209,7 @@ FwdSplit fwd_split(const fa_problem& p) {
 // the shares of dq of a dQ kernel that splits its keys like the forward (0 when it does not)
 size_t dq_share_bytes(const fa_problem& p) {
     const FwdSplit s = fwd_split(p);
-    return s.n_splits <= 1 ? 0 : align256((size_t)s.n_splits * p.B * p.H * p.M * p.D * 2);
+    return s.n_splits <= 1 ? 0 : align256((size_t)s.n_splits * p.B * p.H * p.M * p.D * sizeof(float));
 }
 
 // How dbias is laid out: 0 none, 1 dense (B, H, M, N), 2 reduced in the kernels; -1 = not acceptable
@@ -241,7 +257,7 @@ size_t fa_fwd_workspace_bytes(const fa_problem* p) {
     const FwdSplit s = fwd_split(*p);
     if (s.n_splits <= 1) return 0;
     const size_t rows = (size_t)p->B * p->H * p->M;
-    return align256((size_t)s.n_splits * rows * p->D * 2) + align256((size_t)s.n_splits * rows * sizeof(float));
+    return align256((size_t)s.n_splits * rows * p->D * sizeof(float)) + align256((size_t)s.n_splits * rows * sizeof(float));
 }
 
 int fa_fwd(const fa_fwd_args* a, void* stream) {
@@ -276,7 +292,7 @@ int fa_fwd(const fa_fwd_args* a, void* stream) {
             k.n_splits = s.n_splits;
             k.keys_per_split = s.keys_per_split;
             k.part_o = a->workspace;
-            k.part_lse = reinterpret_cast<float*>(static_cast<char*>(a->workspace) + align256((size_t)s.n_splits * rows * p.D * 2));
+            k.part_lse = reinterpret_cast<float*>(static_cast<char*>(a->workspace) + align256((size_t)s.n_splits * rows * p.D * sizeof(float)));
         }
     }
     // a bias that does not depend on the query row and whose keys fit the kernel's LDS row

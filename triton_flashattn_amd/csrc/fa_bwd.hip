@@ -327,6 +327,27 @@ __global__ __launch_bounds__(256, (StreamCfg<D, stream_kind(BIAS)>::MIN_BLOCKS))
 
     // ---- epilogue: dq = dQ * sm_scale (flash_attention.py:644-646) ----
     ks_.drain();  // K/V slots are dead and no copy is in flight: reuse their LDS for the output tile
+    if (p.dq_splits > 1) {
+        // one of several shares of the keys: into this share's slice of the scratch, in fp32 (the sum
+        // rounds once, like an unsplit run), 16 bytes per lane straight from the accumulators
+        float* pf = reinterpret_cast<float*>(p.part_dq) + (((int64_t)split * p.B * p.H + bh) * M + my_m) * D;
+        if (my_m < M) {
+#pragma unroll
+            for (int db = 0; db < C::DB; db++) {
+#pragma unroll
+                for (int q4 = 0; q4 < 4; q4++) {
+                    const int d = db * 32 + 8 * q4 + 4 * g;
+                    if (d < D) {
+                        f32x4 w;
+#pragma unroll
+                        for (int e = 0; e < 4; e++) w[e] = dq_acc[db][q4 * 4 + e] * p.sm_scale;
+                        *reinterpret_cast<f32x4*>(pf + d) = w;
+                    }
+                }
+            }
+        }
+        return;
+    }
     T* o_lds = reinterpret_cast<T*>(smem) + wave * 32 * OS;
 #pragma unroll
     for (int db = 0; db < C::DB; db++) {
@@ -339,13 +360,10 @@ __global__ __launch_bounds__(256, (StreamCfg<D, stream_kind(BIAS)>::MIN_BLOCKS))
         }
     }
     __syncthreads();
-    const bool shared = p.dq_splits > 1;  // one of several shares of the keys: into this share's slice of the scratch
-    T* op = shared ? reinterpret_cast<T*>(p.part_dq) + ((int64_t)split * p.B * p.H + bh) * M * D
-                   : reinterpret_cast<T*>(p.dq) + (int64_t)b * p.sdq.b + (int64_t)h * p.sdq.h;
-    const int64_t o_stride = shared ? D : p.sdq.s;
+    T* op = reinterpret_cast<T*>(p.dq) + (int64_t)b * p.sdq.b + (int64_t)h * p.sdq.h;
     for (int c = lane; c < 32 * CPR; c += 64) {
         int row = c / CPR, ch = c % CPR;
-        if (mw + row < M) gst16(op + (int64_t)(mw + row) * o_stride + ch * 8, lds_read16(o_lds + row * OS + ch * 8));
+        if (mw + row < M) gst16(op + (int64_t)(mw + row) * p.sdq.s + ch * 8, lds_read16(o_lds + row * OS + ch * 8));
     }
 }
 
@@ -361,9 +379,13 @@ template <typename T, int D> __global__ __launch_bounds__(256) void fa_bwd_dq_su
     if (row >= rows) return;
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     for (int s = 0; s < p.dq_splits; s++) {
-        const T8 v = as_vec<T8>(gld16(reinterpret_cast<const T*>(p.part_dq) + (s * rows + row) * D + c * 8));
+        const float* src = reinterpret_cast<const float*>(p.part_dq) + (s * rows + row) * D + c * 8;
+        const f32x4 lo = *reinterpret_cast<const f32x4*>(src), hi = *reinterpret_cast<const f32x4*>(src + 4);
 #pragma unroll
-        for (int e = 0; e < 8; e++) acc[e] += (float)v[e];
+        for (int e = 0; e < 4; e++) {
+            acc[e] += lo[e];
+            acc[4 + e] += hi[e];
+        }
     }
     const int m = (int)(row % p.M);
     const int64_t bh = row / p.M;

@@ -320,6 +320,27 @@ __global__ __launch_bounds__(256, (StreamCfg<D, fwd_stream_kind(BIAS)>::MIN_BLOC
     if (g == 0 && my_m_late < M) lse_out[my_m_late] = m_i + fast_log2(l_tot);
 
     ks_.drain();  // K/V slots are dead and no copy is in flight: reuse their LDS for the output tile
+    if (shared) {
+        // a share stays in fp32 (the merge rounds once, like an unsplit run): 16 bytes per lane straight
+        // from the accumulators (only problems with few query tiles come here)
+        float* pf = reinterpret_cast<float*>(p.part_o) + (((int64_t)split * p.B * p.H + bh) * M + my_m_late) * D;
+        if (my_m_late < M) {
+#pragma unroll
+            for (int db = 0; db < C::DB; db++) {
+#pragma unroll
+                for (int q4 = 0; q4 < 4; q4++) {
+                    const int d = db * 32 + 8 * q4 + 4 * g;
+                    if (d < D) {
+                        f32x4 w;
+#pragma unroll
+                        for (int e = 0; e < 4; e++) w[e] = o_acc[db][q4 * 4 + e] * inv_l;
+                        *reinterpret_cast<f32x4*>(pf + d) = w;
+                    }
+                }
+            }
+        }
+        return;
+    }
     T* o_lds = reinterpret_cast<T*>(smem) + wave * 32 * OS;
 #pragma unroll
     for (int db = 0; db < C::DB; db++) {
@@ -332,12 +353,10 @@ __global__ __launch_bounds__(256, (StreamCfg<D, fwd_stream_kind(BIAS)>::MIN_BLOC
         }
     }
     __syncthreads();
-    T* op = shared ? reinterpret_cast<T*>(p.part_o) + ((int64_t)split * p.B * p.H + bh) * M * D
-                   : reinterpret_cast<T*>(p.o) + (int64_t)b * p.so.b + (int64_t)h * p.so.h;
-    const int64_t o_stride = shared ? D : p.so.s;
+    T* op = reinterpret_cast<T*>(p.o) + (int64_t)b * p.so.b + (int64_t)h * p.so.h;
     for (int c = lane; c < 32 * CPR; c += 64) {
         int row = c / CPR, ch = c % CPR;
-        if (mw + row < M) gst16(op + (int64_t)(mw + row) * o_stride + ch * 8, lds_read16(o_lds + row * OS + ch * 8));
+        if (mw + row < M) gst16(op + (int64_t)(mw + row) * p.so.s + ch * 8, lds_read16(o_lds + row * OS + ch * 8));
     }
 }
 
@@ -359,9 +378,13 @@ template <typename T, int D> __global__ __launch_bounds__(256) void fa_fwd_merge
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     for (int s = 0; s < p.n_splits; s++) {
         const float w = fast_exp2(p.part_lse[s * rows + row] - lse);
-        const T8 v = as_vec<T8>(gld16(reinterpret_cast<const T*>(p.part_o) + (s * rows + row) * D + c * 8));
+        const float* src = reinterpret_cast<const float*>(p.part_o) + (s * rows + row) * D + c * 8;
+        const f32x4 lo = *reinterpret_cast<const f32x4*>(src), hi = *reinterpret_cast<const f32x4*>(src + 4);
 #pragma unroll
-        for (int e = 0; e < 8; e++) acc[e] += w * (float)v[e];
+        for (int e = 0; e < 4; e++) {
+            acc[e] += w * lo[e];
+            acc[4 + e] += w * hi[e];
+        }
     }
     const int m = (int)(row % p.M);
     const int64_t bh = row / p.M;

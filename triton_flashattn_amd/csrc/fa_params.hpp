@@ -30,8 +30,8 @@ struct FwdParams {
     int bias_vec;  // bias rows may be read with aligned 16-byte loads
     int n_mtiles;
     // Keys split between n_splits work-groups per query tile (1 = no split): split s takes
-    // keys_per_split keys (a multiple of the kernel's step) and writes its output, in the element
-    // type of q, and its LSE to part_o (n_splits, B*H, M, D) / part_lse (n_splits, B*H, M);
+    // keys_per_split keys (a multiple of the kernel's step) and writes its output, in fp32,
+    // and its LSE to part_o (n_splits, B*H, M, D) / part_lse (n_splits, B*H, M);
     // fa_fwd_merge_kernel combines them.
     int n_splits, keys_per_split;
     void* part_o;
@@ -64,8 +64,8 @@ struct BwdParams {
     int bias_vec;   // bias rows may be read with aligned 16-byte loads
     int dbias_vec;  // dbias rows may be written with aligned 16-byte stores
     // dQ kernel: keys split between dq_splits work-groups per query tile (1 = no split), each over
-    // dq_keys_per_split keys, their shares of dq in the element type of q in part_dq (dq_splits,
-    // B*H, M, D); fa_bwd_dq_sum_kernel adds them up
+    // dq_keys_per_split keys, their shares of dq in fp32 in part_dq (dq_splits, B*H, M, D);
+    // fa_bwd_dq_sum_kernel adds them up
     int dq_splits, dq_keys_per_split;
     void* part_dq;
     int row_bias_kind;  // 0, or the element kind (1 bool, 2 fp16, 3 bf16, 4 fp32) of a bias with stride 0 along M:

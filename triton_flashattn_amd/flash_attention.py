@@ -107,9 +107,28 @@ class _HipBackend:
                 raise ValueError("flash_attention: all tensors must be on the same device")
         return dev
 
+    @staticmethod
+    def _check_shapes(q, k, v, lse, bias, alibi, like_q=(), like_k=(), dbias=None):
+        """The kernels take every extent from q and k: whatever else they read or write must agree."""
+        B, M, H, D = q.shape
+        N = k.shape[1]
+        for name, t, want in [("k", k, (B, N, H, D)), ("v", v, (B, N, H, D)), ("lse", lse, (B, H, M))] + \
+                [(n, t, (B, M, H, D)) for n, t in like_q] + [(n, t, (B, N, H, D)) for n, t in like_k]:
+            if t is not None and tuple(t.shape) != want:
+                raise ValueError("%s has shape %s, the kernels need %s" % (name, tuple(t.shape), want))
+        if lse.dtype != torch.float32 or not lse.is_contiguous():
+            raise ValueError("lse must be a dense float32 tensor of shape (B, H, M)")
+        for name, t in (("bias", bias), ("dbias", dbias)):
+            if t is None:
+                continue
+            want = (H,) if alibi else (B, H, M, N)
+            if tuple(t.shape) != want:
+                raise ValueError("%s has shape %s, the kernels need %s" % (name, tuple(t.shape), want))
+
     def fwd(self, q, k, v, bias, causal, sm_scale, o, lse, alibi=False):
         """bias: None, a (B, H, M, N) view (zero strides allowed), or with alibi=True the H slopes."""
         dev = self._require_gpu(q, k, v, bias, o, lse)
+        self._check_shapes(q, k, v, lse, bias, alibi, like_q=[("o", o)])
         lib = _native.load()
         a = _native.FaFwdArgs()
         a.p = self._problem(q, k, bias, causal, sm_scale, alibi)
@@ -145,6 +164,8 @@ class _HipBackend:
         noalloc: call fa_bwd_noalloc (scratch in the library's static device array, nothing is
         allocated; all stages)."""
         dev = self._require_gpu(do, q, k, v, o, bias, lse, dq, dk, dv, dbias)
+        self._check_shapes(q, k, v, lse, bias, alibi, like_q=[("o", o), ("do", do), ("dq", dq)],
+                           like_k=[("dk", dk), ("dv", dv)], dbias=dbias)
         lib = _native.load()
         a = _native.FaBwdArgs()
         a.p = self._problem(q, k, bias, causal, sm_scale, alibi)
@@ -275,7 +296,15 @@ def _bias_rows_ok(b):
     if any(b.shape[i] > 1 and (b.stride(i) * es) % 16 != 0 for i in range(3)):
         return False
     padded = -(-N * es // 16) * 16
-    return N * es == padded or b.stride(2) * es >= padded
+    if N * es == padded:
+        return True
+    if b.stride(2) * es < padded:
+        return False
+    # rows that end inside a 16-byte chunk are fetched to the end of that chunk: the chunk of the very
+    # last row must still lie inside the tensor's storage (true for a column slice of a wider tensor,
+    # not for a view whose last row ends the allocation)
+    last = b.storage_offset() + sum((b.shape[i] - 1) * b.stride(i) for i in range(3))
+    return last * es + padded <= b.untyped_storage().nbytes()
 
 
 def _empty_padded_rows(shape, dtype, device):

@@ -252,11 +252,17 @@ def main():
 
     cfg = make_config("C3", dev)
     B, H, M, N, D = cfg["dims"]
-    # The per-stage timings (events around each stage, repeated) run FIRST: a GPU that has just been
-    # handed over idles at a low clock, and W = 5 warm-up steps (7 ms of work) do not bring it up, so
-    # steps timed right behind them measure the ramp (1.51 ms per step against 1.42 ms once settled).
+    # Order of the measurements.  The first autograd step of a process spends 0.13 s on the host
+    # (engine thread, allocator, library load) with the GPU idle, and an idle GPU drops its clock and
+    # takes some 20 steps (25 ms) to come back: measured per step 1.9, 1.9, 1.8, 1.65, 1.6 ... 1.38 ms.
+    # W = 5 warm-up steps right in front of the timed ones would put that ramp into the timed region.
+    # So: one priming step first (the host-side one-off), then the per-stage timings (events around
+    # each stage, repeated; the first pass is discarded), which leave the clock settled, then the W
+    # warm-up steps and the K timed steps back to back.
+    step(cfg)
+    torch.cuda.synchronize()
     iters = max(5, min(args.steps, 30))
-    time_stages(cfg, iters)  # (discarded: the first pass over the stages is the one that sees the ramp)
+    time_stages(cfg, iters)
     t_fwd, t_bwd, t_main, t_dq = time_stages(cfg, iters)
     for _ in range(args.warmup):
         step(cfg)
@@ -279,7 +285,7 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
-        "order": "per-stage timings first (they settle the clocks), then the warm-up steps, then the timed steps",
+        "order": "one priming step (host-side one-off), per-stage timings (they settle the clock), W warm-up steps, K timed steps",
         "config": {"workload": "BASELINE.json configs[2]: trainable bf16 bias (B,H,M,N), non-causal, "
                                "B=2 H=16 M=N=4096 D=128, flash_attention_fn forward + backward",
                    "B": B, "H": H, "M": M, "N": N, "D": D, "causal": False, "bias": "bf16, requires_grad"},

@@ -705,7 +705,8 @@ __global__ __launch_bounds__((BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>::NT)
     // pointers in scalar registers, one 64-bit add per block, and need no clamps; run_start() points
     // them at the first blocks an interior loop issues.
     // (The kernels that run two work-groups per CU have 128 registers per wave and no room for the
-    // second copy of the loop: they run every step in its general form.)
+    // second copy of the loop: they run every step in its general form.  With their operand reads
+    // left to the compiler they fit, and gain 2 % on the causal D = 64 shape: not worth a second form.)
     constexpr bool IN_LOOPS = !bwd_occ2(D, BIAS);
     const int n_full = M / BMI;  // blocks whose rows all exist
     uint64_t run_rows = 0, run_stat = 0, run_bias = 0;  // Q and LSE (role that issues Q) or dO and delta; bias slices
@@ -856,9 +857,10 @@ __global__ __launch_bounds__((BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>::NT)
         // them into P, so that a step of this role opens with vector work (exponentials) while the
         // partner wave on the same SIMD opens with matrix products, and closes with matrix products
         // while the partner does its vector work.  It needs the Q block one step earlier, i.e. a copy
-        // look-ahead of at least three blocks.  Measured: 6 % on the kernel with a bias (where the
-        // vector work is heaviest), a loss of 4 % without one, which keeps the plain order.
-        constexpr bool S_AHEAD = TB != 0 && C::LA >= 3;
+        // look-ahead of at least three blocks.  Measured: 3 % on the kernel that writes dBias (whose
+        // dP-wave has the most vector work), a loss of 5 % with a bias that is only read and of 4 %
+        // without one, which keep the plain order.
+        constexpr bool S_AHEAD = TB != 0 && C::LA >= 3 && DBIAS == 1;
         f32x16 sacc[NSUB];
         if constexpr (S_AHEAD) {
             T8 a_rows[NR];
@@ -1017,19 +1019,20 @@ __global__ __launch_bounds__((BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>::NT)
         t_in = t_in < t_end ? t_in : t_end;
         t_out = t_out < t_in ? t_in : (t_out < t_end ? t_out : t_end);
         if (!IN_LOOPS) t_in = t_out = t_end;  // one general loop
-        int t = mb_first - 1;
+        // (two passes over ONE copy of the general loop, the interior loop between them)
+        int t = mb_first - 1, stop = t_in;
 #pragma unroll 1
-        for (; t < t_in; t++) s_step(t, std::false_type{});
-        if constexpr (IN_LOOPS) {
-            if (t_in < t_out) {
-                run_start(qp, p.sq.s, lsep, t_in + 1 + C::LA, t_in + 1 + C::LA);
+        for (int pass = 0; pass < (IN_LOOPS ? 2 : 1); pass++) {
 #pragma unroll 1
-                for (; t < t_out; t++) s_step(t, std::true_type{});
+            for (; t < stop; t++) s_step(t, std::false_type{});
+            if constexpr (IN_LOOPS) {
+                if (pass == 0 && t_in < t_out) {
+                    run_start(qp, p.sq.s, lsep, t_in + 1 + C::LA, t_in + 1 + C::LA);
+#pragma unroll 1
+                    for (; t < t_out; t++) s_step(t, std::true_type{});
+                }
             }
-        }
-        if constexpr (IN_LOOPS) {
-#pragma unroll 1
-            for (; t < t_end; t++) s_step(t, std::false_type{});
+            stop = t_end;
         }
         };
         if (TB != 0 && bias_vec) s_loop(std::true_type{});
@@ -1180,19 +1183,20 @@ __global__ __launch_bounds__((BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>::NT)
         t_in = t_in < t_end ? t_in : t_end;
         t_out = t_out < t_in ? t_in : (t_out < t_end ? t_out : t_end);
         if (!IN_LOOPS) t_in = t_out = t_end;  // one general loop
-        int t = mb_first - 1;
+        // (two passes over ONE copy of the general loop, the interior loop between them)
+        int t = mb_first - 1, stop = t_in;
 #pragma unroll 1
-        for (; t < t_in; t++) dp_step(t, std::false_type{});
-        if constexpr (IN_LOOPS) {
-            if (t_in < t_out) {
-                run_start(dop, p.sdo.s, deltap, t_in + C::LA, 0);
+        for (int pass = 0; pass < (IN_LOOPS ? 2 : 1); pass++) {
 #pragma unroll 1
-                for (; t < t_out; t++) dp_step(t, std::true_type{});
+            for (; t < stop; t++) dp_step(t, std::false_type{});
+            if constexpr (IN_LOOPS) {
+                if (pass == 0 && t_in < t_out) {
+                    run_start(dop, p.sdo.s, deltap, t_in + C::LA, 0);
+#pragma unroll 1
+                    for (; t < t_out; t++) dp_step(t, std::true_type{});
+                }
             }
-        }
-        if constexpr (IN_LOOPS) {
-#pragma unroll 1
-            for (; t < t_end; t++) dp_step(t, std::false_type{});
+            stop = t_end;
         }
         };
         if constexpr (DB_VIA_LDS) {

@@ -143,9 +143,30 @@ def test_row_broadcast_bias_is_staged_once_per_work_group(gpu_device, D, kind):
         check(ours, ref, "D%d %s case %d" % (D, kind, i))
 
 
+def test_batch_broadcast_bias_gradient_peaks_at_one_batch_slice(gpu_device):
+    """(1, H, M, N) bias, B = 8: the kernels run one batch at a time into one (1, H, M, N) scratch that is
+    summed into an fp32 accumulator, so the backward never holds a (B, H, M, N) tensor."""
+    B, S, H, D = 8, 1024, 2, 16
+    q, k, v, do, _ = make_inputs(gpu_device, B, S, S, H, D, torch.bfloat16, None, seed=44)
+    bias = torch.randn(1, H, S, S, generator=torch.Generator().manual_seed(44)).bfloat16().to(gpu_device).requires_grad_(True)
+    dense_bytes = B * H * S * S * 2
+    ql, kl, vl = (t.detach().clone().requires_grad_(True) for t in (q, k, v))
+    out = flash_attention_fn(ql, kl, vl, bias, False)
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    before = torch.cuda.memory_allocated()
+    out.backward(do)
+    torch.cuda.synchronize()
+    # scratch (1/8 of dense) + fp32 accumulator (2/8) + the gradient itself (1/8) + dq, dk, dv
+    assert torch.cuda.max_memory_allocated() - before < dense_bytes * 5 // 8
+    ref = run_oracle(q, k, v, do, bias.detach().float().broadcast_to(B, H, S, S), False)
+    ref["dbias"] = ref["dbias"].sum_to_size(1, H, S, S)
+    check({"out": out.detach(), "dq": ql.grad, "dk": kl.grad, "dv": vl.grad, "dbias": bias.grad}, ref, "batch broadcast")
+
+
 def test_batch_or_head_broadcast_bias(gpu_device):
     """A bias broadcast over batches or heads only keeps its (M, N) tiles: read through an expanded
-    view, gradient computed densely and summed over the broadcast dimensions."""
+    view; the gradient is formed one batch at a time and summed in fp32 over the broadcast dimensions."""
     B, M, N, H, D = 2, 200, 264, 3, 64
     for i, shape in enumerate([(1, H, M, N), (B, 1, M, N), (1, 1, M, N), (M, N), (H, M, N)]):
         q, k, v, do, _ = make_inputs(gpu_device, B, M, N, H, D, torch.float16, None, seed=60 + i)

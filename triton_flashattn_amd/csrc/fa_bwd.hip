@@ -529,6 +529,10 @@ __global__ __launch_bounds__((BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>::NT)
     constexpr int BN = C::BN, BMI = C::BMI, CPR = C::CPR, DSS = C::DSS, NSUB = C::NSUB;
     // dBias leaves through the dS tile (16-byte row stores) when it has the element type of dS
     constexpr bool DB_VIA_LDS = DBIAS == 1 && ((BIAS == 2 && __is_same(T, _Float16)) || (BIAS == 3 && __is_same(T, __bf16)));
+    // an fp32 dBias leaves through LDS too, as fp32: the dP-wave turns its part of the P hand-off buffer,
+    // which it has just read and which is not written again before the next step, into a row-major
+    // 32 x 32 tile (4-byte stores, one per element) and stores 16 bytes per lane from there
+    constexpr bool DB_VIA_LDS32 = DBIAS == 1 && BIAS == 4 && BMI == 32;
 
     __shared__ __align__(16) unsigned char smem[C::LDS_BYTES];
 
@@ -1049,16 +1053,23 @@ __global__ __launch_bounds__((BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>::NT)
         // dBias rows that are whole aligned 16-byte chunks leave through unconditional buffer
         // stores (chunks outside the tensor get an offset outside the view): a loop without
         // branches around its stores lets the loads of the next blocks stay in flight across them.
-        const bool db_fast = DB_VIA_LDS && dbias_vec && (N % 8 == 0);
+        const bool db_fast = (DB_VIA_LDS && dbias_vec && (N % 8 == 0)) || (DB_VIA_LDS32 && dbias_vec && (N % 4 == 0));
         __amdgpu_buffer_rsrc_t db_rsrc = make_buffer(nullptr, 0);
         int db_off[2];
-        const int db_row_bytes = DB_VIA_LDS ? (int)p.sdbias.m * 2 : 0;
+        const int db_row_bytes = (DB_VIA_LDS || DB_VIA_LDS32) ? (int)p.sdbias.m * C::ES : 0;
+        // fp32: lane -> row 8 it + lane / 8, keys 4 (lane % 8) .. + 3 of the slice, it = 0 .. 3
+        const int db32_row = lane >> 3, db32_key = 4 * (lane & 7);
         if (db_fast) {
-            db_rsrc = make_buffer(dbp, ((int64_t)(M - 1) * p.sdbias.m + N) * 2);
+            db_rsrc = make_buffer(dbp, ((int64_t)(M - 1) * p.sdbias.m + N) * C::ES);
+            if constexpr (DB_VIA_LDS32) {
+                db_off[0] = nw + db32_key < N ? db32_row * db_row_bytes + (nw + db32_key) * 4 : (int)0x80000000;
+                db_off[1] = 0;
+            } else {
 #pragma unroll
-            for (int it = 0; it < 2; it++) {
-                const int nn = nw + 8 * ((lane >> 5) + 2 * it);
-                db_off[it] = nn < N ? db_row * db_row_bytes + nn * 2 : (int)0x80000000;
+                for (int it = 0; it < 2; it++) {
+                    const int nn = nw + 8 * ((lane >> 5) + 2 * it);
+                    db_off[it] = nn < N ? db_row * db_row_bytes + nn * 2 : (int)0x80000000;
+                }
             }
         }
         float red_acc = 0.f;  // DBIAS == 2: this lane's share of the reduced gradient
@@ -1134,10 +1145,12 @@ __global__ __launch_bounds__((BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>::NT)
                                     red_acc -= dsv * __builtin_fabsf(__builtin_fmaf((float)(m0 + 4 * g) + (float)(ml0 - 4 * g + e), ratio, -(float)my_n));
                                 else red_acc += dsv;
                             }
-                            if constexpr (DBIAS == 1 && !DB_VIA_LDS) {
+                            if constexpr (DBIAS == 1 && !DB_VIA_LDS && !DB_VIA_LDS32) {
                                 const int m = m0 + ml0 + e;
                                 if (m < M && my_n < N) dbp[(int64_t)m * p.sdbias.m + (int64_t)my_n * p.sdbias.n] = (E)dsv;
                             }
+                            // (p_in is this wave's part of the hand-off buffer read at the top of the step)
+                            if constexpr (DB_VIA_LDS32) const_cast<float*>(p_in)[(ml0 + e) * 32 + r] = dsv;
                         }
                         if constexpr (DB_VIA_LDS) *reinterpret_cast<T4*>(ds_lds + r * DSS + ml0) = d4;
                     }
@@ -1165,6 +1178,28 @@ __global__ __launch_bounds__((BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>::NT)
 #pragma unroll
                                 for (int e = 0; e < 8; e++)
                                     if (nn + e < N) dst[(int64_t)e * p.sdbias.n] = __builtin_bit_cast(E, (T)v8[e]);
+                            }
+                        }
+                    }
+                }
+                if constexpr (DB_VIA_LDS32) {
+#pragma unroll
+                    for (int it = 0; it < 4; it++) {
+                        const int row = 8 * it + db32_row;
+                        const f32x4 w = *reinterpret_cast<const f32x4*>(p_in + row * 32 + db32_key);
+                        const i32x4 v = __builtin_bit_cast(i32x4, w);
+                        const int m = m0 + row, nn = nw + db32_key;
+                        if constexpr (DB_FAST) {
+                            const int off = (IN || m < M) ? db_off[0] + (m0 + 8 * it) * db_row_bytes : (int)0x80000000;
+                            buf_store16(db_rsrc, v, off);
+                        } else if (m < M && nn < N) {
+                            float* dst = reinterpret_cast<float*>(dbp) + (int64_t)m * p.sdbias.m + (int64_t)nn * p.sdbias.n;
+                            if (dbias_vec && nn + 4 <= N) {
+                                gst16(dst, v);
+                            } else {
+#pragma unroll
+                                for (int e = 0; e < 4; e++)
+                                    if (nn + e < N) dst[(int64_t)e * p.sdbias.n] = w[e];
                             }
                         }
                     }
@@ -1199,7 +1234,7 @@ __global__ __launch_bounds__((BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>::NT)
             stop = t_end;
         }
         };
-        if constexpr (DB_VIA_LDS) {
+        if constexpr (DB_VIA_LDS || DB_VIA_LDS32) {
             if (db_fast) dp_loop(std::true_type{});
             else dp_loop(std::false_type{});
         } else {

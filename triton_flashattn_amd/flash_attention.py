@@ -394,15 +394,36 @@ def _flash_attn_bwd(do, q, k, v, o, bias, causal, sm_scale, lse, dq, dk, dv, dbi
 def _bias_grad_like(bias, B, H, M, N):
     """(tensor to hand to the kernels, function that turns it into the gradient of `bias`).
     bias is the 4-D view of the caller's bias.  A bias that is broadcast over the query rows gets
-    its gradient reduced in the kernels; one that is only broadcast over batches or heads is
-    computed densely and summed here (an (M, N) accumulator per output slice does not fit the
-    kernels)."""
+    its gradient reduced in the kernels; one that is only broadcast over batches or heads (it keeps
+    its M rows) goes through _bwd_bias_over_batches instead, marked by (None, None)."""
     full = (B, H, M, N)
     if bias.shape[2] == 1 and bias.shape[3] == N:
         return torch.empty(bias.shape, dtype=bias.dtype, device=bias.device), (lambda t: t)
     if tuple(bias.shape) == full:
         return _empty_padded_rows(full, bias.dtype, bias.device), (lambda t: t)
-    return _empty_padded_rows(full, bias.dtype, bias.device), (lambda t: t.sum_to_size(bias.shape))
+    return None, None
+
+
+def _bwd_bias_over_batches(do, q, k, v, o, bias, causal, sm_scale, lse, dq, dk, dv):
+    """The backward for a trainable bias of shape (1 or B, 1 or H, M, N) that is broadcast over
+    batches and / or heads: its gradient is the sum of dS over those dimensions, and a tile of an
+    (M, N) accumulator per output slice does not fit the kernels.  The kernels therefore run one
+    batch at a time, each writing its dS densely into ONE (1, H, M, N) scratch tensor, which is added
+    into an fp32 accumulator of the bias's shape in a fixed order (batches in sequence, heads by a
+    torch sum over a dimension: no atomics): the peak is one batch slice plus the accumulator, not
+    (B, H, M, N), and the sum is formed in fp32 whatever the bias's dtype.  Returns the gradient."""
+    B, M, H, _ = q.shape
+    N = k.shape[1]
+    over_b, over_h = bias.shape[0] == 1, bias.shape[1] == 1
+    acc = torch.zeros(bias.shape, dtype=torch.float32, device=bias.device)
+    scratch = _empty_padded_rows((1, H, M, N), bias.dtype, bias.device)
+    none = lambda t, b: None if t is None else t[b:b + 1]
+    for b in range(B):
+        _flash_attn_bwd(do[b:b + 1], q[b:b + 1], k[b:b + 1], v[b:b + 1], o[b:b + 1], bias[0:1] if over_b else bias[b:b + 1],
+                        causal, sm_scale, lse[b:b + 1], none(dq, b), none(dk, b), none(dv, b), scratch)
+        # (an in-place add of the 16-bit scratch to the fp32 accumulator converts on the fly: no fp32 copy)
+        acc[0 if over_b else b].add_(scratch.sum(dim=1, keepdim=True, dtype=torch.float32)[0] if over_h else scratch[0])
+    return acc.to(bias.dtype)
 
 
 # --------------------------------------------------------------------------------------------
@@ -479,7 +500,10 @@ class FlashAttentionFn(torch.autograd.Function):
                 dbias, finish = torch.empty_like(bias.slopes), (lambda t: t)
         elif ctx.is_bias_trainable:
             dbias, finish = _bias_grad_like(bias, B, H, M, N)
-        if dq is not None or dk is not None or dbias is not None:
+        if ctx.is_bias_trainable and finish is None:
+            dbias = _bwd_bias_over_batches(_pad_head_dim(do, D), q, k, v, o, bias, ctx.causal, ctx.sm_scale, lse, dq, dk, dv)
+            finish = lambda t: t
+        elif dq is not None or dk is not None or dbias is not None:
             _flash_attn_bwd(_pad_head_dim(do, D), q, k, v, o, bias, ctx.causal, ctx.sm_scale, lse, dq, dk, dv, dbias)
         dq = dq if (dq is None or d_qk == D) else dq[..., :d_qk]
         dk = dk if (dk is None or not need_k) else (dk if d_qk == D else dk[..., :d_qk])
@@ -539,8 +563,12 @@ class FlashAttentionQKVPackedFn(torch.autograd.Function):
                 dbias, finish = torch.empty_like(bias.slopes), (lambda t: t)
         elif ctx.is_bias_trainable:
             dbias, finish = _bias_grad_like(bias, B, H, S, S)
-        if dqkv is not None or dbias is not None:
-            g = (None, None, None) if dqkv is None else (dqkv[:, :, 0], dqkv[:, :, 1], dqkv[:, :, 2])
+        g = (None, None, None) if dqkv is None else (dqkv[:, :, 0], dqkv[:, :, 1], dqkv[:, :, 2])
+        if ctx.is_bias_trainable and finish is None:
+            dbias = _bwd_bias_over_batches(do, qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], o, bias, ctx.causal, ctx.sm_scale,
+                                           lse, g[0], g[1], g[2])
+            finish = lambda t: t
+        elif dqkv is not None or dbias is not None:
             _flash_attn_bwd(do, qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], o, bias, ctx.causal, ctx.sm_scale, lse,
                             g[0], g[1], g[2], dbias)
         dbias = None if dbias is None else finish(dbias)
@@ -621,7 +649,10 @@ def _op_bwd(do: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
         b4 = _bias_kernel_layout(b4)
     if bias_grad:
         dbias, finish = _bias_grad_like(b4, B, H, M, k.shape[1])
-    _flash_attn_bwd(do, q, k, v, o, b4, causal, sm_scale, lse, dq, dk, dv, dbias)
+    if bias_grad and finish is None:
+        dbias, finish = _bwd_bias_over_batches(do, q, k, v, o, b4, causal, sm_scale, lse, dq, dk, dv), (lambda t: t)
+    else:
+        _flash_attn_bwd(do, q, k, v, o, b4, causal, sm_scale, lse, dq, dk, dv, dbias)
     # an operator cannot return None: no bias gradient is an empty tensor
     return dq, dk, dv, (finish(dbias).reshape(bias.shape).contiguous() if bias_grad else q.new_empty((0,)))
 

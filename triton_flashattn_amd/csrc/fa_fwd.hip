@@ -274,7 +274,11 @@ __global__ __launch_bounds__(256, (StreamCfg<D, fwd_stream_kind(BIAS)>::MIN_BLOC
             }
             l_i += rs;  // per-lane partial sum; the two halves of a row are added at the end
         };
-        if constexpr (STEP_MASKED) {
+        if constexpr (STEP_MASKED && D > 128) {
+            // (head dim 256: one form of the softmax step in the edge loop; a second copy of the
+            // 32 matrix products of a block there costs the registers that the interior loops need)
+            softmax_step(std::true_type{});
+        } else if constexpr (STEP_MASKED) {
             if (need_mask || !(qk_scale > 0.f)) softmax_step(std::true_type{});
             else softmax_step(std::false_type{});
         } else {

@@ -308,6 +308,11 @@ __global__ __launch_bounds__(256, (StreamCfg<D, stream_kind(BIAS)>::MIN_BLOCKS))
     if (!(qk_scale > 0.f) || m0 + BM > M) n_fast = 0;
     auto run = [&](auto bv_tag) {
         constexpr bool BV = decltype(bv_tag)::value;
+        // The loads of this lane's rows issued above are the compiler's own.  Left in flight, they would
+        // make it wait for "all vector-memory operations" at their first use inside EVERY step of the
+        // loops (it cannot know that they land once), and that wait drains the queue of copies issued
+        // steps ahead.  Waiting for them here, before the first copy, keeps the loops free of it.
+        wait_vmcnt<0>();
         ks_.template prologue<BV>();
         // the leading fast steps whose copies stay inside the tensors issue them without clamps
         const int n_lean = (BV || TB == 0) ? ks_.lean_steps(n_fast, m0 + BM) : 0;

@@ -136,7 +136,9 @@ size_t fa_bwd_workspace_bytes(const fa_problem *p);
  * their softmaxes (the outputs of the shares in fp32, and their LSEs); 0 when the
  * problem has enough query tiles to fill the GPU, or is causal.  No counterpart in the reference (its grid is one program
  * per query tile, flash_attention.py:666).  The workspace is optional: without it fa_fwd runs one
- * work-group per query tile, with the same results up to fp32 rounding of the merge. */
+ * work-group per query tile, with the same results up to fp32 rounding of the merge.  "Enough" is
+ * measured against the compute units of the CURRENT device (as is the dq part of
+ * fa_bwd_workspace_bytes): ask with the device current on which fa_fwd / fa_bwd will run. */
 size_t fa_fwd_workspace_bytes(const fa_problem *p);
 
 /* Enqueue the backward (delta, dK/dV/dBias/dQ) on `stream`.

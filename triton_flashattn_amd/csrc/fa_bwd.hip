@@ -1132,6 +1132,7 @@ __global__ __launch_bounds__((BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>::NT)
                 // ---- dS = P (dP - delta) (flash_attention.py:303-308) ----
 #pragma unroll
                 for (int sb = 0; sb < NSUB; sb++) {
+                    i32x2 pk_even = {0, 0};
 #pragma unroll
                     for (int q4 = 0; q4 < 4; q4++) {
                         const int ml0 = sb * 32 + 8 * q4 + 4 * g;
@@ -1142,7 +1143,6 @@ __global__ __launch_bounds__((BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>::NT)
                         for (int e = 0; e < 4; e++) {
                             const int i = q4 * 4 + e;
                             const float dsv = p4[e] * (sacc[sb][i] - del4[e]);
-                            op_cur[sb][i >> 3][i & 7] = (T)dsv;
                             d4[e] = (T)dsv;
                             if constexpr (DBIAS == 2) {
                                 // rows past M and keys past N have P = 0 exactly, hence dS = 0
@@ -1157,6 +1157,12 @@ __global__ __launch_bounds__((BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>::NT)
                             // (p_in is this wave's part of the hand-off buffer read at the top of the step)
                             if constexpr (DB_VIA_LDS32) const_cast<float*>(p_in)[(ml0 + e) * 32 + r] = dsv;
                         }
+                        // the operand of the dK product is made of the same packed words that go to the dS
+                        // tile (assembled as integers: element-wise inserts made the compiler convert
+                        // every value a second time, one by one, and merge the halves with permutes)
+                        const i32x2 pk = __builtin_bit_cast(i32x2, d4);
+                        if (q4 & 1) op_cur[sb][q4 >> 1] = __builtin_bit_cast(T8, (i32x4){pk_even[0], pk_even[1], pk[0], pk[1]});
+                        else pk_even = pk;
                         if constexpr (DB_VIA_LDS) *reinterpret_cast<T4*>(ds_lds + r * DSS + ml0) = d4;
                     }
                 }

@@ -135,6 +135,9 @@ __global__ __launch_bounds__(256, (StreamCfg<D, stream_kind(BIAS)>::MIN_BLOCKS))
     }
 
     const float qk_scale = p.sm_scale * kLog2e;
+    // bool mask, unmasked steps: the two values that the offset of a score's exponent can take (the lane
+    // is one query row), so that an element costs a select and not a select and a subtraction
+    const float neg_lse = 0.f - lse_i, mask_lse = kMask - lse_i;
     f32x16 dq_acc[C::DB];  // dQ^T: rows = head dim, column = my_m
 #pragma unroll
     for (int db = 0; db < C::DB; db++)
@@ -271,7 +274,7 @@ __global__ __launch_bounds__(256, (StreamCfg<D, stream_kind(BIAS)>::MIN_BLOCKS))
                         } else if constexpr (BIAS == 0) {
                             pv = fast_exp2(__builtin_fmaf(s[i], qk_scale, -lse_i));
                         } else if constexpr (BIAS == 1) {
-                            pv = fast_exp2(__builtin_fmaf(s[i], qk_scale, (keep[e] ? 0.f : kMask) - lse_i));
+                            pv = fast_exp2(__builtin_fmaf(s[i], qk_scale, keep[e] ? neg_lse : mask_lse));
                         } else if constexpr (BOOLROW) {
                             pv = fast_exp2(__builtin_fmaf(s[i], qk_scale, bv[e] - lse_i));
                         } else {
@@ -950,7 +953,9 @@ __global__ __launch_bounds__((BwdCfg<D, tile_kind(BIAS), bwd_occ2(D, BIAS)>::NT)
                                     x = __fadd_rn(x, __fadd_rn(tmask, add));
                                     pv = fast_exp2(x - lse4[e]);
                                 } else {
-                                    const float off = NATURAL ? __builtin_fmaf(bv, kLog2e, -lse4[e]) : bv - lse4[e];
+                                    // (without a bias the offset is the negated LSE itself: written as 0 - lse it
+                                    // would cost a subtraction per element, +0 - x not being -x)
+                                    const float off = BIAS == 0 ? -lse4[e] : (NATURAL ? __builtin_fmaf(bv, kLog2e, -lse4[e]) : bv - lse4[e]);
                                     pv = fast_exp2(__builtin_fmaf(sacc[sb][i], qk_scale, off));
                                 }
                                 p4[e] = pv;

@@ -118,6 +118,19 @@ def test_sm_scale_and_untrainable_bias(gpu_device):
     check(ours, run_oracle(q, k, v, do, bias, False, 0.05))
 
 
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("bias_kind", [None, "bool", "bf16", "f32"])
+def test_head_dim_128_without_bias_gradient(gpu_device, bias_kind, causal):
+    """The kernels of head dim 128 that write no dBias (no bias, a mask, a float bias nobody differentiates)
+    on tiles long enough for their steady-state loops: the backward of these interleaves its matrix and
+    vector work differently from the kernel that writes dBias."""
+    for M, N in ((640, 640), (1056, 1056) if causal else (1056, 520)):
+        q, k, v, do, bias = make_inputs(gpu_device, 1, M, N, 2, 128, torch.bfloat16, bias_kind, seed=M + N, trainable=False)
+        ours = run_ours(q, k, v, do, bias, causal)
+        assert ours["dbias"] is None
+        check(ours, run_oracle(q, k, v, do, bias, causal), "D128 %s causal=%s %s" % (bias_kind, causal, (M, N)))
+
+
 def test_lse_is_log2_sum_exp(gpu_device):
     q, k, v, do, bias = make_inputs(gpu_device, 2, 300, 170, 3, 128, torch.bfloat16, "f32", trainable=False)
     o, lse = _flash_attn_fwd(q, k, v, bias, False, 0.1)

@@ -145,8 +145,10 @@ size_t fa_fwd_workspace_bytes(const fa_problem *p);
  * Replaces _flash_attn_bwd, flash_attention.py:688-763 (K and bias pre-scale :699-704 included). */
 int fa_bwd(const fa_bwd_args *args, void *stream);
 
-/* The three stages fa_bwd enqueues, in order.  fa_bwd(args, stream) is
- * fa_bwd_stages(args, stream, FA_STAGE_ALL). */
+/* The three stages of the backward.  fa_bwd(args, stream) is fa_bwd_stages(args, stream, FA_STAGE_ALL).
+ * They are enqueued in this order, except that a dQ stage which does not read dbias (see below) is
+ * enqueued first when FA_STAGE_PREP is asked for in the same call: its kernel then forms delta itself,
+ * bit for bit as the delta pass would, and stores it for the dK/dV kernel, and no delta pass is launched. */
 enum fa_bwd_stage {
     FA_STAGE_PREP = 1, /* delta = rowsum(o * do)          (flash_attention.py:197-233) */
     FA_STAGE_MAIN = 2, /* dK, dV, dBias over key tiles    (flash_attention.py:237-454) */

@@ -156,6 +156,35 @@ def test_stages_one_by_one_equal_one_call(gpu_device, bias_dtype):
     assert torch.equal(alone[1], whole[1]) and torch.equal(alone[2], whole[2])
 
 
+@pytest.mark.parametrize("D", [16, 32, 64, 128, 256])
+def test_delta_formed_by_the_dq_kernel_equals_the_delta_pass(gpu_device, D):
+    """Without a dBias to read, the dQ kernel runs first and forms delta = rowsum(o * do) itself when delta and
+    dQ are asked for in one call.  What it stores (the dK/dV kernel reads it) is bit for bit the delta of the
+    separate pass, and so are all gradients of the two orders."""
+    S = _native
+    B, M, N, H = 2, 200, 264, 3
+    g = torch.Generator(device="cpu").manual_seed(D)
+    mk = lambda *s: torch.randn(*s, generator=g).bfloat16().to(gpu_device)
+    q, k, v, do = mk(B, M, H, D), mk(B, N, H, D), mk(B, N, H, D), mk(B, M, H, D)
+    scale = D ** -0.5
+    o, lse = _flash_attn_fwd(q, k, v, None, False, scale)
+    res = []
+    for stage_list in ([S.FA_STAGE_PREP, S.FA_STAGE_MAIN, S.FA_STAGE_DQ], [S.FA_STAGE_ALL], [S.FA_STAGE_PREP | S.FA_STAGE_DQ, S.FA_STAGE_MAIN]):
+        dq, dk, dv = torch.full_like(q, 7.0), torch.full_like(k, 7.0), torch.full_like(v, 7.0)
+        ws = fa_mod._backend.bwd_workspace(q, k, None, False, scale)
+        ws.fill_(0xff)
+        for st in stage_list:
+            fa_mod._backend.bwd(do, q, k, v, o, None, False, scale, lse, dq, dk, dv, None, stages=st, workspace=ws)
+        torch.cuda.synchronize()
+        delta = ws[: B * H * M * 4].view(torch.float32).clone()
+        res.append((delta, dq, dk, dv))
+    ref = (o.float() * do.float()).sum(-1).permute(0, 2, 1).reshape(-1)   # (B, H, M)
+    assert torch.allclose(res[0][0], ref, atol=1e-3, rtol=1e-4)
+    for other in res[1:]:
+        for name, a, b_ in zip(("delta", "dq", "dk", "dv"), res[0], other):
+            assert torch.equal(a, b_), (D, name)
+
+
 def test_dq_routes_agree(gpu_device):
     """dQ from the dBias just written (one product) against dQ recomputed from q, k, v and the bias
     (three products; taken when dBias rows are not whole 16-byte chunks, here N = 324... odd rows)."""

@@ -17,6 +17,9 @@
 namespace fa {
 
 // ---------------------------------------------------------------------------------------------
+// delta of one row: every 16-byte chunk c of the row is summed element by element with fused
+// multiply-adds, then the D / 8 chunk sums are added pairwise, c with c ^ w for w = D / 16, ..., 2, 1.
+// (fa_bwd_dq_kernel forms the same sums in the same order when it stands in for this kernel.)
 template <typename T, int D>
 __global__ __launch_bounds__(256) void fa_bwd_prep_kernel(const BwdParams p) {
     constexpr int LPR = D / 8;         // lanes per row (16 bytes each)
@@ -35,7 +38,7 @@ __global__ __launch_bounds__(256) void fa_bwd_prep_kernel(const BwdParams p) {
         T8 ov = as_vec<T8>(gld16(op + c * 8));
         T8 dv = as_vec<T8>(gld16(dp + c * 8));
 #pragma unroll
-        for (int e = 0; e < 8; e++) acc += (float)ov[e] * (float)dv[e];
+        for (int e = 0; e < 8; e++) acc = __builtin_fmaf((float)ov[e], (float)dv[e], acc);
     }
 #pragma unroll
     for (int w = LPR / 2; w >= 1; w >>= 1) acc += __shfl_xor(acc, w, 64);
@@ -125,7 +128,31 @@ __global__ __launch_bounds__(256, (StreamCfg<D, stream_kind(BIAS)>::MIN_BLOCKS))
     float lse_i = 0.f, delta_i = 0.f;
     if (!FROM_DS && my_m < M) {
         lse_i = p.lse[((int64_t)b * p.H + h) * M + my_m];
-        delta_i = p.delta[((int64_t)b * p.H + h) * M + my_m];
+        if (!p.dq_makes_delta) delta_i = p.delta[((int64_t)b * p.H + h) * M + my_m];
+    }
+    if (!FROM_DS && p.dq_makes_delta) {
+        // This kernel runs first and forms delta = sum_d o * do itself (flash_attention.py:215-227), in the
+        // order of fa_bwd_prep_kernel: this lane holds the chunks 2 ks + g of its row (dO^T above), sums
+        // each with fused multiply-adds, adds chunk c to chunk c ^ w for w = D / 16, ..., 2 (both in this
+        // lane) and last to chunk c ^ 1 (in the lane of the other g).  The dK/dV kernel reads what is stored.
+        const T* op = reinterpret_cast<const T*>(p.o) + (int64_t)b * p.so.b + (int64_t)h * p.so.h;
+        float part[C::KSTEPS];
+#pragma unroll
+        for (int ks = 0; ks < C::KSTEPS; ks++) {
+            i32x4 ro = {0, 0, 0, 0};
+            if (my_m < M) ro = gld16(op + (int64_t)my_m * p.so.s + ks * 16 + 8 * g);
+            const T8 ov = as_vec<T8>(ro);
+            float a = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; e++) a = __builtin_fmaf((float)ov[e], (float)doreg[ks][e], a);
+            part[ks] = a;
+        }
+#pragma unroll
+        for (int hs = C::KSTEPS / 2; hs >= 1; hs >>= 1)
+#pragma unroll
+            for (int ks = 0; ks < hs; ks++) part[ks] = part[ks] + part[ks + hs];
+        delta_i = part[0] + __shfl_xor(part[0], 32, 64);
+        if (g == 0 && my_m < M && split == 0) p.delta[((int64_t)b * p.H + h) * M + my_m] = delta_i;
     }
 
     int n_steps = (N + BK - 1) / BK;
@@ -1360,9 +1387,66 @@ template <typename T, int D> static hipError_t launch_all(const BwdParams& p, in
     const int64_t rows = (int64_t)p.B * p.H * p.M;
     dim3 rgrid((unsigned)((rows + RPB - 1) / RPB));
     hipError_t e = hipSuccess;
-    if (stages & 1) {
+    // dBias in fp32 or in the element type of q, written densely a moment ago by the key-tile kernel
+    // in rows of whole 16-byte chunks, is the dS the dQ product needs.  Only when that kernel ran in
+    // this very call (or the caller vouches for the contents of dbias, bit 8) is it read.
+    constexpr int DS_BIAS = __is_same(T, _Float16) ? 2 : 3;
+    const bool ds_valid = dbias == 1 && ((stages & 2) || (stages & 8));
+    const bool from_ds = (stages & 4) && ds_valid && (bias == DS_BIAS || bias == 4) && p.dbias_vec;
+    // A dQ kernel that recomputes dS depends on nothing but delta.  When delta and dQ are asked for in one
+    // call it runs FIRST and forms delta itself, bit for bit as fa_bwd_prep_kernel would, which saves a
+    // launch and a pass over o and do; the dK/dV kernel then reads the delta it has stored.
+    const bool dq_first = (stages & 5) == 5 && !from_ds;
+    auto launch_dq = [&](bool makes_delta) -> hipError_t {
+        // the one-product form runs at the rate of the dS stream and gains nothing from more work-groups
+        BwdParams pq = p;
+        pq.dq_makes_delta = makes_delta ? 1 : 0;
+        if (from_ds) pq.dq_splits = 1;
+        dim3 qgrid((unsigned)(pq.n_mtiles * pq.dq_splits * pq.B * pq.H));
+        if (from_ds && bias == DS_BIAS) {
+            if (causal) hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, DS_BIAS, true, true>), qgrid, dim3(256), 0, st, pq);
+            else hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, DS_BIAS, false, true>), qgrid, dim3(256), 0, st, pq);
+        } else if (from_ds && bias == 4) {
+            if (causal) hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, 4, true, true>), qgrid, dim3(256), 0, st, pq);
+            else hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, 4, false, true>), qgrid, dim3(256), 0, st, pq);
+        } else {
+#define FA_CASE(BK)                                                                                               \
+    case BK:                                                                                                      \
+        if (causal) hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, BK, true>), qgrid, dim3(256), 0, st, pq);           \
+        else hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, BK, false>), qgrid, dim3(256), 0, st, pq);                 \
+        break;
+            // a bias without a row dimension whose keys (of one share) fit the LDS row is staged once per
+            // work-group instead of streamed
+            const int keys_per_wg = pq.dq_splits > 1 ? pq.dq_keys_per_split : pq.N;
+            const int qbias = (p.row_bias_kind != 0 && keys_per_wg <= kRowBiasKeys) ? (p.row_bias_kind == 1 ? 7 : 6) : bias;
+            switch (qbias) {
+                FA_CASE(0)
+                FA_CASE(1)
+                FA_CASE(2)
+                FA_CASE(3)
+                FA_CASE(4)
+                FA_CASE(5)
+                FA_CASE(6)
+                FA_CASE(7)
+                default: return hipErrorInvalidValue;
+            }
+#undef FA_CASE
+        }
+        hipError_t eq = hipGetLastError();
+        if (eq == hipSuccess && pq.dq_splits > 1) {
+            const int64_t threads = (int64_t)p.B * p.H * p.M * (D / 8);
+            hipLaunchKernelGGL((fa_bwd_dq_sum_kernel<T, D>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, pq);
+            eq = hipGetLastError();
+        }
+        return eq;
+    };
+    if ((stages & 1) && !dq_first) {
         hipLaunchKernelGGL((fa_bwd_prep_kernel<T, D>), rgrid, dim3(256), 0, st, p);
         e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    if (dq_first) {
+        e = launch_dq(true);
         if (e != hipSuccess) return e;
     }
     if (stages & 2) {
@@ -1404,53 +1488,7 @@ template <typename T, int D> static hipError_t launch_all(const BwdParams& p, in
             if (e != hipSuccess) return e;
         }
     }
-    if (stages & 4) {
-        // dBias in fp32 or in the element type of q, written densely a moment ago by the key-tile kernel
-        // in rows of whole 16-byte chunks, is the dS the dQ product needs.  Only when that kernel ran in
-        // this very call (or the caller vouches for the contents of dbias, bit 8) is it read.
-        constexpr int DS_BIAS = __is_same(T, _Float16) ? 2 : 3;
-        const bool ds_valid = dbias == 1 && ((stages & 2) || (stages & 8));
-        const bool from_ds = ds_valid && (bias == DS_BIAS || bias == 4) && p.dbias_vec;
-        // the one-product form runs at the rate of the dS stream and gains nothing from more work-groups
-        BwdParams pq = p;
-        if (from_ds) pq.dq_splits = 1;
-        dim3 qgrid((unsigned)(pq.n_mtiles * pq.dq_splits * pq.B * pq.H));
-        if (ds_valid && bias == DS_BIAS && p.dbias_vec) {
-            if (causal) hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, DS_BIAS, true, true>), qgrid, dim3(256), 0, st, pq);
-            else hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, DS_BIAS, false, true>), qgrid, dim3(256), 0, st, pq);
-        } else if (ds_valid && bias == 4 && p.dbias_vec) {
-            if (causal) hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, 4, true, true>), qgrid, dim3(256), 0, st, pq);
-            else hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, 4, false, true>), qgrid, dim3(256), 0, st, pq);
-        } else {
-#define FA_CASE(BK)                                                                                               \
-    case BK:                                                                                                      \
-        if (causal) hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, BK, true>), qgrid, dim3(256), 0, st, pq);           \
-        else hipLaunchKernelGGL((fa_bwd_dq_kernel<T, D, BK, false>), qgrid, dim3(256), 0, st, pq);                 \
-        break;
-        // a bias without a row dimension whose keys (of one share) fit the LDS row is staged once per
-        // work-group instead of streamed
-        const int keys_per_wg = pq.dq_splits > 1 ? pq.dq_keys_per_split : pq.N;
-        const int qbias = (p.row_bias_kind != 0 && keys_per_wg <= kRowBiasKeys) ? (p.row_bias_kind == 1 ? 7 : 6) : bias;
-        switch (qbias) {
-            FA_CASE(0)
-            FA_CASE(1)
-            FA_CASE(2)
-            FA_CASE(3)
-            FA_CASE(4)
-            FA_CASE(5)
-            FA_CASE(6)
-            FA_CASE(7)
-            default: return hipErrorInvalidValue;
-        }
-#undef FA_CASE
-        }
-        e = hipGetLastError();
-        if (e == hipSuccess && pq.dq_splits > 1) {
-            const int64_t threads = (int64_t)p.B * p.H * p.M * (D / 8);
-            hipLaunchKernelGGL((fa_bwd_dq_sum_kernel<T, D>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, pq);
-            e = hipGetLastError();
-        }
-    }
+    if ((stages & 4) && !dq_first) e = launch_dq(false);
     return e;
 }
 

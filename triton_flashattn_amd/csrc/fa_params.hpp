@@ -70,6 +70,8 @@ struct BwdParams {
     void* part_dq;
     int row_bias_kind;  // 0, or the element kind (1 bool, 2 fp16, 3 bf16, 4 fp32) of a bias with stride 0 along M:
                         // the dK/dV kernel reads it as one value per key, the dQ kernel stages it in LDS
+    int dq_makes_delta; // the dQ kernel runs before the dK/dV kernel and forms delta itself (and stores it),
+                        // in place of fa_bwd_prep_kernel and bit for bit like it
 };
 
 }  // namespace fa
